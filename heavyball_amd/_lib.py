@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbstep.so")
 
 # include/hbstep.h
-ABI_VERSION = 4  # HB_ABI_VERSION this binding was written against
+ABI_VERSION = 5  # HB_ABI_VERSION this binding was written against
 FMT_F32, FMT_BF16, FMT_F16, FMT_ECC_BF16_8, FMT_ECC_BF16_16, FMT_ECC_F16_8, FMT_ECC_F16_16 = range(7)
 ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD = 1, 2, 4, 8, 16, 32, 64
@@ -20,6 +20,7 @@ RNG_HALF, RNG_PHILOX = 0, 1
 STREAM_MARS_SR, STREAM_OLD_GRAD, STREAM_EXP_AVG, STREAM_EXP_AVG_SQ, STREAM_PARAM, STREAM_INIT_PARAM, STREAM_NS_INPUT = range(7)
 STREAM_CLIP, STREAM_EXP_AVG_SLOW = 8, 9
 NS_LEGACY, NS_BF16_UPDATE = 1, 2
+NOALLOC_MAX_TENSORS = 65536  # HB_NOALLOC_MAX_TENSORS
 GEMM_ACCUMULATE, GEMM_SYMMETRIC = 1, 2
 MOM_NESTEROV_EMA, MOM_EMA, MOM_HEAVYBALL, MOM_NESTEROV_HEAVYBALL = range(4)
 
@@ -73,6 +74,7 @@ class HbStepDesc(Structure):
 
 _PROTOTYPES = {
     "hb_fused_step": (ctypes.c_int, [POINTER(HbStepDesc), c_void_p]),
+    "hb_fused_step_noalloc": (ctypes.c_int, [POINTER(HbStepDesc), c_void_p]),
     "hb_update_param": (ctypes.c_int, [POINTER(HbStepDesc), c_void_p]),
     "hb_ecc_encode": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_uint64, c_uint32, c_uint32, c_int64, c_void_p]),
     "hb_ecc_decode": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p]),

@@ -116,7 +116,7 @@ static bool fmt_ok_state(int f) { return f == HB_FMT_F32 || f == HB_FMT_BF16 || 
 static bool fmt_ok_grad(int f) { return f == HB_FMT_F32 || f == HB_FMT_BF16 || f == HB_FMT_F16; }
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states) {
+static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states, bool need_counts = true) {
   if (!d) return set_error(HB_EINVAL, "null descriptor");
   if (d->n_chunks < 0 || d->n_tensors < 0) return set_error(HB_EINVAL, "negative sizes");
   if (!d->offsets || !d->numel || !d->chunks) return set_error(HB_EINVAL, "offsets, numel and chunks are required");
@@ -133,7 +133,7 @@ static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states) {
     if ((d->grad == nullptr) == (d->grad_ptrs == nullptr)) return set_error(HB_EINVAL, "exactly one of grad / grad_ptrs must be set");
     if (d->grad && !aligned16(d->grad)) return set_error(HB_EINVAL, "grad slab must be 16-byte aligned");
   }
-  if (caution && !d->caution_count) return set_error(HB_EINVAL, "caution_count scratch required with HB_FLAG_CAUTION");
+  if (caution && need_counts && !d->caution_count) return set_error(HB_EINVAL, "caution_count scratch required with HB_FLAG_CAUTION");
   if (need_states) {
     if (d->algo < HB_ALGO_ADAM || d->algo > HB_ALGO_NADAM) return set_error(HB_EINVAL, "bad algo");
     if ((d->flags & HB_FLAG_ADOPT_WARMUP) && (d->algo != HB_ALGO_ADOPT || caution || (d->flags & HB_FLAG_UPDATE_ONLY)))
@@ -201,24 +201,70 @@ static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states) {
 
 }  // namespace hb
 
-extern "C" int hb_fused_step(const HbStepDesc* d, void* stream_) {
-  using namespace hb;
-  StepArgs a;
-  if (int rc = fill_args(d, a, true)) return rc;
-  if (d->n_chunks == 0) return HB_OK;
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
+namespace hb {
+
+// Both entry points of the fused step.  `counts`: the per-tensor caution counters the two caution launches share
+// (zeroed here by a fill kernel, not by hipMemsetAsync, so that a caller may capture the call in a graph).
+static int run_fused_step(const HbStepDesc* d, StepArgs& a, uint32_t* counts, hipStream_t stream, const char* what) {
   const bool mars = (d->flags & HB_FLAG_MARS) != 0;
   const bool caution = (d->flags & HB_FLAG_CAUTION) != 0;
   const int grid = persistent_grid(d->n_chunks);
   if (grid <= 0) return set_error(HB_ELAUNCH, "could not query the device");
+  a.counts = counts;
   if (caution) {
-    zero_u32_kernel<<<(d->n_tensors + 255) / 256, 256, 0, stream>>>(d->caution_count, d->n_tensors);
+    zero_u32_kernel<<<(d->n_tensors + 255) / 256, 256, 0, stream>>>(counts, d->n_tensors);
     pick_kernel(d->algo, mars, kCautionCount, a.pf, a.gf, a.sf)<<<grid, kThreads, 0, stream>>>(a);
     pick_kernel(d->algo, mars, kCautionApply, a.pf, a.gf, a.sf)<<<grid, kThreads, 0, stream>>>(a);
   } else {
     pick_kernel(d->algo, mars, kNoCaution, a.pf, a.gf, a.sf)<<<grid, kThreads, 0, stream>>>(a);
   }
-  return check_launch("hb_fused_step");
+  return check_launch(what);
+}
+
+// Scratch of hb_fused_step_noalloc: the caution counters live in the library's own device memory.  Every device the
+// library runs on holds its own copy of this array at its own address, for the life of the process.
+static __device__ __align__(256) uint32_t scratch[HB_NOALLOC_MAX_TENSORS];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<uint32_t*> g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device, resolved once
+
+// The device address of `scratch` on the current device.  The array's name is only a host-side handle: what kernels
+// and fills are given is the address hipGetSymbolAddress reports for the device that is current.
+static int scratch_of_current_device(uint32_t** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return set_error(HB_ELAUNCH, "hb_fused_step_noalloc: no current device");
+  uint32_t* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return set_error(HB_ELAUNCH, "hb_fused_step_noalloc: hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // concurrent first calls resolve the same address
+  }
+  *out = ptr;
+  return HB_OK;
+}
+
+}  // namespace hb
+
+extern "C" int hb_fused_step(const HbStepDesc* d, void* stream_) {
+  using namespace hb;
+  StepArgs a;
+  if (int rc = fill_args(d, a, true, true)) return rc;
+  if (d->n_chunks == 0) return HB_OK;
+  return run_fused_step(d, a, d->caution_count, static_cast<hipStream_t>(stream_), "hb_fused_step");
+}
+
+extern "C" int hb_fused_step_noalloc(const HbStepDesc* d, void* stream_) {
+  using namespace hb;
+  StepArgs a;
+  if (int rc = fill_args(d, a, true, false)) return rc;
+  if (d->n_tensors > HB_NOALLOC_MAX_TENSORS)
+    return set_error(HB_EINVAL, "hb_fused_step_noalloc: %d tensors, the built-in scratch holds counters for at most %d", d->n_tensors,
+                     HB_NOALLOC_MAX_TENSORS);
+  if (d->n_chunks == 0) return HB_OK;
+  uint32_t* counts = nullptr;
+  if (int rc = scratch_of_current_device(&counts)) return rc;
+  return run_fused_step(d, a, counts, static_cast<hipStream_t>(stream_), "hb_fused_step_noalloc");
 }
 
 extern "C" int hb_update_param(const HbStepDesc* d, void* stream_) {

@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 4
+#define HB_ABI_VERSION 5
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -150,6 +150,16 @@ typedef struct HbStepDesc {
  * (:3616-3627), the caution mask (:3652-3658), the parameter update (:2373-2390) and the ECC / stochastic-rounding
  * writes (:1288-1324, :2341-2370) */
 int hb_fused_step(const HbStepDesc* desc, void* stream);
+
+/* hb_fused_step for callers that cannot allocate device memory or hand over a scratch buffer: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * descriptor and results as hb_fused_step, except that `caution_count` is ignored (it may be NULL): the per-tensor
+ * caution counters live in a device array inside the library (4 * HB_NOALLOC_MAX_TENSORS bytes on every GPU the
+ * library runs on, held until the process ends).  More than HB_NOALLOC_MAX_TENSORS tensors: HB_EINVAL.  The call
+ * allocates and frees nothing and clears the counters it uses with a fill kernel.  Every call on one GPU shares that
+ * GPU's array, so two calls with HB_FLAG_CAUTION that overlap on one GPU (different streams or threads) race. */
+#define HB_NOALLOC_MAX_TENSORS 65536
+int hb_fused_step_noalloc(const HbStepDesc* desc, void* stream);
 
 /* chain()'s non-fused tail, update_param_ (heavyball/utils.py:2393-2406): p <- p*(1 - decay*lr) + u*(-lr) on a slab,
  * with `update` an fp32 slab at the same offsets.  Uses param/param_corr/param_fmt, offsets, numel, chunks, flags
