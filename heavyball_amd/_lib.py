@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbstep.so")
 
 # include/hbstep.h
-ABI_VERSION = 5  # HB_ABI_VERSION this binding was written against
+ABI_VERSION = 6  # HB_ABI_VERSION this binding was written against
 FMT_F32, FMT_BF16, FMT_F16, FMT_ECC_BF16_8, FMT_ECC_BF16_16, FMT_ECC_F16_8, FMT_ECC_F16_16 = range(7)
 ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD = 1, 2, 4, 8, 16, 32, 64

@@ -39,7 +39,8 @@ __global__ void sr_bf16_kernel(const float* __restrict__ src, uint16_t* __restri
 
 __global__ void philox_words_kernel(uint32_t* out, int64_t n, uint64_t q0, Rng rng, uint32_t stream_id) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
-    const Rand8 r = rng.octet((int64_t)((q0 + (uint64_t)i) << 3), stream_id);
+    const Rand8 r = rng.mode == HB_RNG_PHILOX ? rng.call((int64_t)((q0 + (uint64_t)i) << 2), stream_id)
+                                               : Rand8{{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u}};
     out[4 * i + 0] = r.w[0];
     out[4 * i + 1] = r.w[1];
     out[4 * i + 2] = r.w[2];

@@ -29,8 +29,10 @@ extern template StepKernel pick_algo<HB_ALGO_NADAM>(bool, int, int, int, int);
 
 // chain()'s non-fused tail (heavyball/utils.py:2393-2406): the update is an fp32 slab (in a.m), optional caution
 // against the gradient.  COUNT = 1 only counts masked elements.
+constexpr int kUThreads = 256;                           // update_param_kernel: one workgroup per chunk,
+constexpr int kUGroups = HB_CHUNK / (kUThreads * 8);     // kUGroups octets per lane
 template <int CAUTION, int PF>
-__global__ __launch_bounds__(kThreads) void update_param_kernel(const StepArgs a) {
+__global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs a) {
   const int pf = PF == kDyn ? a.pf : PF;
   constexpr bool kCount = CAUTION == kCautionCount;
   const bool cautious_wd = (a.flags & HB_FLAG_CAUTIOUS_WD) != 0;
@@ -53,8 +55,8 @@ __global__ __launch_bounds__(kThreads) void update_param_kernel(const StepArgs a
     }
     uint32_t masked = 0;
 #pragma unroll
-    for (int k = 0; k < kGroups; ++k) {
-      const int e = k * (kThreads * 8) + threadIdx.x * 8;
+    for (int k = 0; k < kUGroups; ++k) {
+      const int e = k * (kUThreads * 8) + threadIdx.x * 8;
       if (e >= valid) continue;
       const int64_t idx = flat0 + e;
       Raw ru, rp;
@@ -208,7 +210,7 @@ namespace hb {
 static int run_fused_step(const HbStepDesc* d, StepArgs& a, uint32_t* counts, hipStream_t stream, const char* what) {
   const bool mars = (d->flags & HB_FLAG_MARS) != 0;
   const bool caution = (d->flags & HB_FLAG_CAUTION) != 0;
-  const int grid = persistent_grid(d->n_chunks);
+  const int grid = persistent_grid(d->n_chunks * kSub);
   if (grid <= 0) return set_error(HB_ELAUNCH, "could not query the device");
   a.counts = counts;
   if (caution) {
@@ -278,12 +280,12 @@ extern "C" int hb_update_param(const HbStepDesc* d, void* stream_) {
   if (grid <= 0) return set_error(HB_ELAUNCH, "could not query the device");
   if (caution) {
     zero_u32_kernel<<<(d->n_tensors + 255) / 256, 256, 0, stream>>>(d->caution_count, d->n_tensors);
-    update_param_kernel<kCautionCount, kDyn><<<grid, kThreads, 0, stream>>>(a);
-    update_param_kernel<kCautionApply, kDyn><<<grid, kThreads, 0, stream>>>(a);
+    update_param_kernel<kCautionCount, kDyn><<<grid, kUThreads, 0, stream>>>(a);
+    update_param_kernel<kCautionApply, kDyn><<<grid, kUThreads, 0, stream>>>(a);
   } else if (a.pf == HB_FMT_F32) {
-    update_param_kernel<kNoCaution, HB_FMT_F32><<<grid, kThreads, 0, stream>>>(a);
+    update_param_kernel<kNoCaution, HB_FMT_F32><<<grid, kUThreads, 0, stream>>>(a);
   } else {
-    update_param_kernel<kNoCaution, kDyn><<<grid, kThreads, 0, stream>>>(a);
+    update_param_kernel<kNoCaution, kDyn><<<grid, kUThreads, 0, stream>>>(a);
   }
   return check_launch("hb_update_param");
 }

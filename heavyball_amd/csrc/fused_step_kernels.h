@@ -9,12 +9,28 @@
 
 namespace hb {
 
+// Work decomposition of the step kernel: every lane owns HB_EPL consecutive elements of each role per group, a workgroup
+// of HB_THREADS lanes takes kWork = HB_THREADS * HB_EPL * HB_GROUPS consecutive elements, and a chunk of the chunk table
+// is kSub such work units.  Measured on MI355X: the narrower the run of a lane, the closer the kernel gets to the
+// bandwidth of a plain copy (an arithmetic-free kernel with the access pattern of the ECC LaProp step moves 5.8 TB/s with
+// 8 elements per lane, 6.0 with 4, 6.3 with 2), and one group per lane beats two (all loads of a wavefront are in flight
+// at once with few registers, so more wavefronts fit and reads and writes alternate at a finer grain).
 #ifndef HB_THREADS
 #define HB_THREADS 256
 #endif
+#ifndef HB_GROUPS
+#define HB_GROUPS 1
+#endif
+#ifndef HB_EPL
+#define HB_EPL 4
+#endif
 constexpr int kThreads = HB_THREADS;
-constexpr int kGroups = HB_CHUNK / (kThreads * 8);
-static_assert(kGroups * kThreads * 8 == HB_CHUNK, "chunk must be a whole number of octet groups");
+constexpr int kGroups = HB_GROUPS;
+constexpr int kE = HB_EPL;
+constexpr int kWork = kThreads * kE * kGroups;
+constexpr int kSub = HB_CHUNK / kWork;
+static_assert(kE == 2 || kE == 4 || kE == 8, "2, 4 or 8 elements per lane");
+static_assert(kSub >= 1 && kSub * kWork == HB_CHUNK, "a chunk must be a whole number of work units");
 
 struct StepArgs {
   char* param;
@@ -50,7 +66,7 @@ __device__ __forceinline__ void for_each_index(F&& f, std::integer_sequence<int,
   (f(std::integral_constant<int, K>{}), ...);
 }
 
-// One chunk.  FULL = every lane's octets are inside the tensor (the common case): no bounds tests at all.
+// One work unit.  FULL = every lane's elements are inside the tensor (the common case): no bounds tests at all.
 template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF, bool FULL>
 __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, const int gf, const int sf, const int t, const int valid,
                                            const int64_t flat0, const char* gbase, const int64_t g0, const bool g_slab, const float scale,
@@ -72,23 +88,23 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   // sqrt(v) is clamped to eps: with eps >= 1e-18 a denormal v (root < 1.1e-19) never reaches the result
   const bool fast_sqrt = a.eps >= 1e-18f;
 
-  Raw rp[kGroups], rg[kGroups], rm[kGroups], rv[kGroups], ro[kGroups], rs[kGroups];
-  float gtail[kGroups][8];
+  RawT<kE> rp[kGroups], rg[kGroups], rm[kGroups], rv[kGroups], ro[kGroups], rs[kGroups];
+  float gtail[kGroups][kE];
   bool tail[kGroups];
 #pragma unroll
   for (int k = 0; k < kGroups; ++k) {
-    const int e = k * (kThreads * 8) + threadIdx.x * 8;
+    const int e = k * (kThreads * kE) + threadIdx.x * kE;
     tail[k] = false;
     if (FULL || e < valid) {
       const int64_t idx = flat0 + e;
-      if (FULL || g_slab || e + 8 <= valid) {
+      if (FULL || g_slab || e + kE <= valid) {
         raw_load<GF>(rg[k], gf, gbase, nullptr, g0 + e);
-      } else {  // last, partial octet of a gradient that is not padded: element loads
+      } else {  // last, partial run of a gradient that is not padded: element loads
         tail[k] = true;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) gtail[k][j] = e + j < valid ? load_elem(gbase, gf, g0 + e + j) : 0.0f;
+        for (int j = 0; j < kE; ++j) gtail[k][j] = e + j < valid ? load_elem(gbase, gf, g0 + e + j) : 0.0f;
       }
-      if (kAdopt) rm[k] = rp[k] = Raw{};
+      if (kAdopt) rm[k] = rp[k] = RawT<kE>{};
       if (!kAdopt || !warmup) raw_load<SF>(rm[k], sf, a.m, a.m_corr, idx);
       if (kNeedV) raw_load<SF>(rv[k], sf, a.v, a.v_corr, idx);
       if (kMix) raw_load<SF>(rs[k], sf, a.s3, a.s3_corr, idx);
@@ -98,17 +114,17 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   }
 
   uint32_t masked = 0;
-  // One octet group.  A generic lambda over a compile-time index instead of an unrolled loop: with run-time format codes
+  // One group.  A generic lambda over a compile-time index instead of an unrolled loop: with run-time format codes
   // the body is too large for the unroller, and a rolled loop would index the register arrays above dynamically.
   auto group = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
-    const int e = k * (kThreads * 8) + threadIdx.x * 8;
+    const int e = k * (kThreads * kE) + threadIdx.x * kE;
     if (!FULL && e >= valid) return;
     const int64_t idx = flat0 + e;
-    float p[8], g[8], m[8], v[8], og[8], u[8], sl[8];
+    float p[kE], g[kE], m[kE], v[kE], og[kE], u[kE], sl[kE];
     if (!FULL && tail[k]) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) g[j] = gtail[k][j];
+      for (int j = 0; j < kE; ++j) g[j] = gtail[k][j];
     } else {
       raw_decode<GF>(rg[k], gf, g);
     }
@@ -119,10 +135,10 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
 
     if (MARS) {
       raw_decode<SF>(ro[k], sf, og);
-      Rand8 rn;
-      if (gf == HB_FMT_BF16) rn = a.rng.octet(idx, HB_STREAM_MARS_SR);
+      Noise<kE> rn{}, rn_og{};  // streams HB_STREAM_MARS_SR and HB_STREAM_OLD_GRAD share their Philox calls
+      if (gf == HB_FMT_BF16 || (og_rounds && !kCount)) a.rng.noise_pair<kE>(idx, HB_STREAM_MARS_SR >> 1, rn, rn_og);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kE; ++j) {
         float gc = g[j] * a.omamars + og[j] * a.amars;  // heavyball/utils.py:1048
         if (gf == HB_FMT_BF16) gc = bf16_to_f32(sr_bf16(gc, rn.bits16(j)));
         else if (gf == HB_FMT_F16) gc = f16_to_f32(f32_to_f16_rne(gc));
@@ -130,47 +146,54 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
         g[j] = gc;
       }
       if (!kCount) {
-        Raw w;
-        Rand8 rn_og;
-        if (og_rounds) rn_og = a.rng.octet(idx, HB_STREAM_OLD_GRAD);
-        else rn_og = Rand8{{0, 0, 0, 0}};
+        RawT<kE> w;
+        if (!og_rounds) rn_og = Noise<kE>{};
         raw_encode<SF>(w, sf, og, rn_og);
         raw_store<SF>(w, sf, a.og, a.og_corr, idx);
         if (write_grad) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
+          for (int j = 0; j < kE; ++j)
             if (FULL || e + j < valid) store_elem(const_cast<char*>(gbase), gf, g0 + e + j, g[j]);
         }
       }
     }
 
+    // The denominators of the group first, with one wave-uniform choice of the square-root routine for all of them
+    // (taken per element the choice costs two branches each).
+    float den[kE];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kE; ++j) {
       if (kNadam && coupled) g[j] = __builtin_fmaf(p[j], a.wd, g[j]);  // heavyball/utils.py:363-364, add_ with alpha
-      float den = 1.0f;
-      if (kAdopt) {  // heavyball/utils.py:2300-2304: the denominator comes from v as the steps before left it
-        const float root = fast_sqrt ? sqrt_rn_normal(v[j]) : __builtin_sqrtf(v[j]);
-        den = __builtin_fmaxf(root, a.eps);
-        v[j] = v[j] * a.oma2 + (g[j] * g[j]) * a.a2;
-      } else if (kNeedV) {
-        v[j] = v[j] * a.oma2 + (g[j] * g[j]) * a.a2;  // heavyball/utils.py:426-427
-        const float root = fast_sqrt ? sqrt_rn_normal(v[j]) : __builtin_sqrtf(v[j]);
-        den = __builtin_fmaxf(root, a.eps);  // heavyball/utils.py:413-414
+      // heavyball/utils.py:426-427; ADOPT (:2300-2304) takes the denominator from v as the steps before left it
+      if (kNeedV && !kAdopt) v[j] = v[j] * a.oma2 + (g[j] * g[j]) * a.a2;
+      den[j] = 1.0f;
+    }
+    if (kNeedV || kAdopt) {
+      if (fast_sqrt) {
+#pragma unroll
+        for (int j = 0; j < kE; ++j) den[j] = max_nonnan(sqrt_rn_normal(v[j]), a.eps);  // heavyball/utils.py:413-414
+      } else {
+#pragma unroll
+        for (int j = 0; j < kE; ++j) den[j] = max_nonnan(__builtin_sqrtf(v[j]), a.eps);
       }
+    }
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      if (kAdopt) v[j] = v[j] * a.oma2 + (g[j] * g[j]) * a.a2;
       if (ALGO == HB_ALGO_ADAM) {
         m[j] = m[j] * a.oma1 + g[j] * a.a1;  // heavyball/utils.py:1939
-        u[j] = kNeedV ? m[j] / den : m[j];   // :1943 (count pass: the sign of m is the sign of m / den)
+        u[j] = kNeedV ? m[j] / den[j] : m[j];   // :1943 (count pass: the sign of m is the sign of m / den)
       } else if (kMix) {
         m[j] = m[j] * a.oma1 + g[j] * a.a1;     // heavyball/utils.py:2104 (fast)
         sl[j] = sl[j] * a.oma3 + g[j] * a.a3;   // :2105 (slow, beta3 is not debiased)
         const float num = m[j] + sl[j] * a.alpha;  // :2108
-        u[j] = kNeedV ? num / den : num;
+        u[j] = kNeedV ? num / den[j] : num;
       } else if (kNadam) {
         m[j] = m[j] * a.oma1 + g[j] * a.a1;              // heavyball/utils.py:394 (beta1 is not debiased)
-        u[j] = (g[j] / den) * gw + (m[j] / den) * ew;    // :409
+        u[j] = (g[j] / den[j]) * gw + (m[j] / den[j]) * ew;    // :409
         if (coupled) u[j] = u[j] - p[j] * a.wd;          // :378
       } else {  // LaProp, and ADOPT with the denominator chosen above
-        m[j] = m[j] * a.oma1 + (g[j] / den) * a.a1;  // heavyball/utils.py:2267-2268, :2300
+        m[j] = m[j] * a.oma1 + (g[j] / den[j]) * a.a1;  // heavyball/utils.py:2267-2268, :2300
         u[j] = m[j];
       }
       if (CAUTION != kNoCaution) {
@@ -186,34 +209,33 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
     if (!kCount) {
       if (update_only) {  // un-fused transform: the update itself is the output
 #pragma unroll
-        for (int j = 0; j < 8; ++j) p[j] = u[j];
+        for (int j = 0; j < kE; ++j) p[j] = u[j];
       } else if (cautious_wd) {  // heavyball/utils.py:2388-2389
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kE; ++j) {
           const float om = ((f2u(p[j]) ^ f2u(u[j])) >> 31) ? 1.0f : a.omdl;
           p[j] = p[j] * om + u[j] * a.neg_lr;
         }
       } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) p[j] = p[j] * a.omdl + u[j] * a.neg_lr;  // heavyball/utils.py:2389
+        for (int j = 0; j < kE; ++j) p[j] = p[j] * a.omdl + u[j] * a.neg_lr;  // heavyball/utils.py:2389
       }
-      Raw w;
-      Rand8 rn;
+      RawT<kE> w;
+      Noise<kE> rn_m{}, rn_v{};  // exp_avg and exp_avg_sq share their Philox calls
+      if (state_rounds) a.rng.noise_pair<kE>(idx, HB_STREAM_EXP_AVG >> 1, rn_m, rn_v);
       if (!kAdopt || !warmup) {
-        rn = state_rounds ? a.rng.octet(idx, HB_STREAM_EXP_AVG) : Rand8{{0, 0, 0, 0}};
-        raw_encode<SF>(w, sf, m, rn);
+        raw_encode<SF>(w, sf, m, rn_m);
         raw_store<SF>(w, sf, a.m, a.m_corr, idx);
       }
-      rn = state_rounds ? a.rng.octet(idx, HB_STREAM_EXP_AVG_SQ) : Rand8{{0, 0, 0, 0}};
-      raw_encode<SF>(w, sf, v, rn);
+      raw_encode<SF>(w, sf, v, rn_v);
       raw_store<SF>(w, sf, a.v, a.v_corr, idx);
       if (kMix) {
-        rn = state_rounds ? a.rng.octet(idx, HB_STREAM_EXP_AVG_SLOW) : Rand8{{0, 0, 0, 0}};
+        const Noise<kE> rn = state_rounds ? a.rng.noise<kE>(idx, HB_STREAM_EXP_AVG_SLOW) : Noise<kE>{};
         raw_encode<SF>(w, sf, sl, rn);
         raw_store<SF>(w, sf, a.s3, a.s3_corr, idx);
       }
       if (!kAdopt || !warmup) {
-        rn = pf != HB_FMT_F32 ? a.rng.octet(idx, HB_STREAM_PARAM) : Rand8{{0, 0, 0, 0}};
+        const Noise<kE> rn = pf != HB_FMT_F32 ? a.rng.noise<kE>(idx, HB_STREAM_PARAM) : Noise<kE>{};
         raw_encode<PF>(w, pf, p, rn);
         raw_store<PF>(w, pf, a.param, a.param_corr, idx);
       }
@@ -232,14 +254,15 @@ __global__ __launch_bounds__(kThreads) void fused_step_kernel(const StepArgs a) 
   const int pf = PF == kDyn ? a.pf : PF;
   const int gf = GF == kDyn ? a.gf : GF;
   const int sf = SF == kDyn ? a.sf : SF;
-  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
-    const int2 ent = a.chunks[c];
+  for (int64_t w = blockIdx.x; w < a.n_chunks * kSub; w += gridDim.x) {
+    const int2 ent = a.chunks[w / kSub];
     const int t = ent.x;
     const int64_t off = a.offsets[t];
     const int64_t n = a.numel[t];
-    const int64_t local0 = (int64_t)ent.y * HB_CHUNK;
+    const int64_t local0 = (int64_t)ent.y * HB_CHUNK + (int64_t)(w % kSub) * kWork;
     const int64_t rem = n - local0;
-    const int valid = rem < HB_CHUNK ? (int)rem : HB_CHUNK;
+    if (rem <= 0) continue;  // a work unit behind the end of the tensor's last chunk
+    const int valid = rem < kWork ? (int)rem : kWork;
     const int64_t flat0 = off + local0;
     const bool g_slab = a.grad_ptrs == nullptr;
     const char* gbase = g_slab ? a.grad : a.grad_ptrs[t];
@@ -255,7 +278,7 @@ __global__ __launch_bounds__(kThreads) void fused_step_kernel(const StepArgs a) 
       gw = a.tscal[2 * t];
       ew = a.tscal[2 * t + 1];
     }
-    if (valid == HB_CHUNK) step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, true>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
+    if (valid == kWork) step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, true>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
     else step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, false>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
   }
 }

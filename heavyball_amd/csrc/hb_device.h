@@ -25,10 +25,20 @@ __device__ __forceinline__ float f16_to_f32(uint32_t h) { return (float)__builti
 __device__ __forceinline__ uint32_t f32_to_f16_rne(float x) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x); }
 
 // ---------------------------------------------------------------------------------------------------------
-// Philox4x32-10 (Salmon et al., SC'11).  One call yields 128 bits = 16 bits for each element of an octet.
+// Philox4x32-10 (Salmon et al., SC'11).  One call yields 128 bits: 16 bits for each of the 4 elements of a quartet
+// (4 consecutive elements, flat index a multiple of 4), for the two rounding sites of a stream pair:
+//   counter = (q lo, q hi, step, stream >> 1) with q = flat_index >> 2,  key = seed
+//   element j = flat_index & 3 of stream s takes word (s & 1) * 2 + (j >> 1), low half if j is even else high half.
+// exp_avg (2) and exp_avg_sq (3) share a call, so a lane that owns a quartet needs one call for both moments.
 // ---------------------------------------------------------------------------------------------------------
-struct Rand8 {
+struct Rand8 {  // the four words of one call; also: the noise of an octet for one stream (two calls, see Rng::octet)
   uint32_t w[4];
+  __device__ __forceinline__ uint32_t bits16(int j) const { return (w[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu; }
+};
+// noise of E consecutive elements for one stream: 16 bits each, element j in word j >> 1
+template <int E>
+struct Noise {
+  uint32_t w[E / 2];
   __device__ __forceinline__ uint32_t bits16(int j) const { return (w[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu; }
 };
 
@@ -53,13 +63,66 @@ __device__ __forceinline__ Rand8 philox4x32_10(uint32_t c0, uint32_t c1, uint32_
 struct Rng {
   uint32_t seed_lo, seed_hi, step;
   int mode;
-  // noise for the octet whose first element has flat slab index `flat` (a multiple of 8)
-  __device__ __forceinline__ Rand8 octet(int64_t flat, uint32_t stream) const {
-    if (mode == HB_RNG_PHILOX) {
-      uint64_t q = (uint64_t)flat >> 3;
-      return philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), step, stream, seed_lo, seed_hi);
+  // the call that serves the quartet holding flat index `flat` for the stream pair `pair` (= stream >> 1)
+  __device__ __forceinline__ Rand8 call(int64_t flat, uint32_t pair) const {
+    const uint64_t q = (uint64_t)flat >> 2;
+    return philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), step, pair, seed_lo, seed_hi);
+  }
+  // noise of the E elements starting at flat index `flat` (a multiple of E; E = 2, 4 or 8) for both streams of a
+  // pair: `even` for stream 2 * pair, `odd` for stream 2 * pair + 1
+  template <int E>
+  __device__ __forceinline__ void noise_pair(int64_t flat, uint32_t pair, Noise<E>& even, Noise<E>& odd) const {
+    static_assert(E == 2 || E == 4 || E == 8, "2, 4 or 8 elements per lane");
+#pragma unroll
+    for (int i = 0; i < E / 2; ++i) even.w[i] = odd.w[i] = 0x80008000u;
+    if (mode != HB_RNG_PHILOX) return;
+    const Rand8 r = call(flat, pair);
+    if constexpr (E == 2) {  // half a quartet: the lanes of both halves make the same call and take their word
+      const bool hi = (flat & 2) != 0;
+      even.w[0] = hi ? r.w[1] : r.w[0];
+      odd.w[0] = hi ? r.w[3] : r.w[2];
+    } else {  // written out per quartet: a loop over the quartets is left rolled and indexes the words through scratch
+      even.w[0] = r.w[0];
+      even.w[1] = r.w[1];
+      odd.w[0] = r.w[2];
+      odd.w[1] = r.w[3];
+      if constexpr (E == 8) {
+        const Rand8 r2 = call(flat + 4, pair);
+        even.w[2] = r2.w[0];
+        even.w[3] = r2.w[1];
+        odd.w[2] = r2.w[2];
+        odd.w[3] = r2.w[3];
+      }
     }
-    return Rand8{{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u}};
+  }
+  template <int E>
+  __device__ __forceinline__ Noise<E> noise(int64_t flat, uint32_t stream) const {
+    static_assert(E == 2 || E == 4 || E == 8, "2, 4 or 8 elements per lane");
+    Noise<E> out;
+#pragma unroll
+    for (int i = 0; i < E / 2; ++i) out.w[i] = 0x80008000u;
+    if (mode == HB_RNG_PHILOX) {
+      const bool second = (stream & 1) != 0;
+      const Rand8 r = call(flat, stream >> 1);
+      if constexpr (E == 2) {
+        const uint32_t lo = second ? r.w[2] : r.w[0], hi = second ? r.w[3] : r.w[1];
+        out.w[0] = (flat & 2) ? hi : lo;
+      } else {
+        out.w[0] = second ? r.w[2] : r.w[0];
+        out.w[1] = second ? r.w[3] : r.w[1];
+        if constexpr (E == 8) {
+          const Rand8 r2 = call(flat + 4, stream >> 1);
+          out.w[2] = second ? r2.w[2] : r2.w[0];
+          out.w[3] = second ? r2.w[3] : r2.w[1];
+        }
+      }
+    }
+    return out;
+  }
+  // noise for the octet whose first element has flat slab index `flat` (a multiple of 8), one stream
+  __device__ __forceinline__ Rand8 octet(int64_t flat, uint32_t stream) const {
+    const Noise<8> n = noise<8>(flat, stream);
+    return Rand8{{n.w[0], n.w[1], n.w[2], n.w[3]}};
   }
 };
 
@@ -154,12 +217,14 @@ __device__ __forceinline__ uint32_t pack_bytes(int c0, int c1, int c2, int c3) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Octets: every lane owns 8 consecutive elements of each role
+// Runs of E consecutive elements per lane (E = 8: octet, 4: quartet, 2: pair) of each role
 // ---------------------------------------------------------------------------------------------------------
-struct Raw {  // what the loads of one role bring in, before decoding
-  uint4 a, b;  // F32: a,b = 8 floats; 16-bit primaries: a = 8 halves
-  uint4 c;     // corrections: int8 -> c.x,c.y ; int16 -> c
+template <int E>
+struct RawT {          // what the loads of one role bring in, before decoding
+  uint32_t a[E];       // F32: E floats; 16-bit primaries: E / 2 words
+  uint32_t c[E / 2];   // corrections: int8 -> E / 4 words (E = 2: the low half of c[0]); int16 -> E / 2 words
 };
+using Raw = RawT<8>;
 
 __host__ __device__ __forceinline__ constexpr bool fmt_is_ecc(int f) { return f >= HB_FMT_ECC_BF16_8; }
 __host__ __device__ __forceinline__ constexpr bool fmt_prim_bf16(int f) {
@@ -169,38 +234,93 @@ __host__ __device__ __forceinline__ constexpr bool fmt_corr8(int f) { return f =
 __host__ __device__ __forceinline__ constexpr int fmt_prim_bytes(int f) { return f == HB_FMT_F32 ? 4 : 2; }
 __host__ __device__ __forceinline__ constexpr int fmt_corr_bytes(int f) { return !fmt_is_ecc(f) ? 0 : (fmt_corr8(f) ? 1 : 2); }
 
-template <int F>
-__device__ __forceinline__ void raw_load_s(Raw& r, const char* prim, const char* corr, int64_t idx) {
-  if (F == HB_FMT_F32) {
-    const uint4* p = reinterpret_cast<const uint4*>(prim + idx * 4);
-    r.a = p[0];
-    r.b = p[1];
+// Accesses of the slab, BYTES = 2 .. 32 per lane.  HB_NT = 1 marks them nontemporal: every byte of the slab is touched
+// exactly once per step, so nothing is gained by keeping it in the caches.
+#ifndef HB_NT
+#define HB_NT 1
+#endif
+typedef uint32_t hb_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t hb_u32x2 __attribute__((ext_vector_type(2)));
+template <typename T>
+__device__ __forceinline__ T ld_as(const char* p) {
+#if HB_NT
+  return __builtin_nontemporal_load(reinterpret_cast<const T*>(p));
+#else
+  return *reinterpret_cast<const T*>(p);
+#endif
+}
+template <typename T>
+__device__ __forceinline__ void st_as(char* p, T v) {
+#if HB_NT
+  __builtin_nontemporal_store(v, reinterpret_cast<T*>(p));
+#else
+  *reinterpret_cast<T*>(p) = v;
+#endif
+}
+template <int BYTES>
+__device__ __forceinline__ void ld_slab(const char* p, uint32_t* d) {
+  static_assert(BYTES == 2 || BYTES == 4 || BYTES == 8 || BYTES == 16 || BYTES == 32, "access width");
+  if constexpr (BYTES == 2) {
+    d[0] = ld_as<uint16_t>(p);
+  } else if constexpr (BYTES == 4) {
+    d[0] = ld_as<uint32_t>(p);
+  } else if constexpr (BYTES == 8) {
+    const hb_u32x2 v = ld_as<hb_u32x2>(p);
+    d[0] = v.x;
+    d[1] = v.y;
   } else {
-    r.a = *reinterpret_cast<const uint4*>(prim + idx * 2);
-    if (fmt_is_ecc(F)) {
-      if (fmt_corr8(F)) {
-        uint2 t = *reinterpret_cast<const uint2*>(corr + idx);
-        r.c.x = t.x;
-        r.c.y = t.y;
-      } else {
-        r.c = *reinterpret_cast<const uint4*>(corr + idx * 2);
-      }
+#pragma unroll
+    for (int h = 0; h < BYTES / 16; ++h) {
+      const hb_u32x4 v = ld_as<hb_u32x4>(p + 16 * h);
+      d[4 * h] = v.x;
+      d[4 * h + 1] = v.y;
+      d[4 * h + 2] = v.z;
+      d[4 * h + 3] = v.w;
+    }
+  }
+}
+template <int BYTES>
+__device__ __forceinline__ void st_slab(char* p, const uint32_t* d) {
+  static_assert(BYTES == 2 || BYTES == 4 || BYTES == 8 || BYTES == 16 || BYTES == 32, "access width");
+  if constexpr (BYTES == 2) {
+    st_as<uint16_t>(p, (uint16_t)d[0]);
+  } else if constexpr (BYTES == 4) {
+    st_as<uint32_t>(p, d[0]);
+  } else if constexpr (BYTES == 8) {
+    const hb_u32x2 v = {d[0], d[1]};
+    st_as<hb_u32x2>(p, v);
+  } else {
+#pragma unroll
+    for (int h = 0; h < BYTES / 16; ++h) {
+      const hb_u32x4 v = {d[4 * h], d[4 * h + 1], d[4 * h + 2], d[4 * h + 3]};
+      st_as<hb_u32x4>(p + 16 * h, v);
     }
   }
 }
 
-template <int F>
-__device__ __forceinline__ void raw_decode_s(const Raw& r, float (&x)[8]) {
+template <int F, int E>
+__device__ __forceinline__ void raw_load_s(RawT<E>& r, const char* prim, const char* corr, int64_t idx) {
   if (F == HB_FMT_F32) {
-    x[0] = u2f(r.a.x); x[1] = u2f(r.a.y); x[2] = u2f(r.a.z); x[3] = u2f(r.a.w);
-    x[4] = u2f(r.b.x); x[5] = u2f(r.b.y); x[6] = u2f(r.b.z); x[7] = u2f(r.b.w);
+    ld_slab<4 * E>(prim + idx * 4, r.a);
+  } else {
+    ld_slab<2 * E>(prim + idx * 2, r.a);
+    if (fmt_is_ecc(F)) {
+      if (fmt_corr8(F)) ld_slab<E>(corr + idx, r.c);
+      else ld_slab<2 * E>(corr + idx * 2, r.c);
+    }
+  }
+}
+
+template <int F, int E>
+__device__ __forceinline__ void raw_decode_s(const RawT<E>& r, float (&x)[E]) {
+  if (F == HB_FMT_F32) {
+#pragma unroll
+    for (int j = 0; j < E; ++j) x[j] = u2f(r.a[j]);
     return;
   }
-  const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
-  const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    uint32_t h = (w[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
+  for (int j = 0; j < E; ++j) {
+    uint32_t h = (r.a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
     if (F == HB_FMT_BF16) {
       x[j] = bf16_to_f32(h);
     } else if (F == HB_FMT_F16) {
@@ -208,40 +328,46 @@ __device__ __forceinline__ void raw_decode_s(const Raw& r, float (&x)[8]) {
     } else {
       int c;
       if (fmt_corr8(F)) {
-        c = (int)(int8_t)((cw[j >> 2] >> ((j & 3) * 8)) & 0xFFu);
+        c = (int)(int8_t)((r.c[j >> 2] >> ((j & 3) * 8)) & 0xFFu);
       } else {
-        c = (int)(int16_t)((cw[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu);
+        c = (int)(int16_t)((r.c[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu);
       }
       x[j] = ecc_decode<fmt_prim_bf16(F), fmt_corr8(F)>(h, c);
     }
   }
 }
 
-// encode 8 fp32 values into the storage format; `rnd` supplies the 16 noise bits of each element
-template <int F>
-__device__ __forceinline__ void raw_encode_s(Raw& r, const float (&x)[8], const Rand8& rnd) {
+// encode E fp32 values into the storage format; `rnd` supplies the 16 noise bits of each element
+template <int F, int E>
+__device__ __forceinline__ void raw_encode_s(RawT<E>& r, const float (&x)[E], const Noise<E>& rnd) {
   if (F == HB_FMT_F32) {
-    r.a = make_uint4(f2u(x[0]), f2u(x[1]), f2u(x[2]), f2u(x[3]));
-    r.b = make_uint4(f2u(x[4]), f2u(x[5]), f2u(x[6]), f2u(x[7]));
+#pragma unroll
+    for (int j = 0; j < E; ++j) r.a[j] = f2u(x[j]);
     return;
   }
-  uint32_t w[4] = {0, 0, 0, 0};
-  uint32_t cw[4] = {0, 0, 0, 0};
+  uint32_t w[E / 2];
+  uint32_t cw[E / 2];
+#pragma unroll
+  for (int i = 0; i < E / 2; ++i) w[i] = cw[i] = 0;
   if (F == HB_FMT_ECC_BF16_8) {
     // hot format: convert in pairs, keep the primaries packed, take exponent and value straight from the packed word
-    int c[8];
+    int c[E];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < E / 2; ++q) {
       const uint32_t pk = pack_bf16_rne(x[2 * q], x[2 * q + 1]);
       w[q] = pk;
       c[2 * q] = ecc_correction<true, true>(x[2 * q], pk & 0xFFFFu, rnd.w[q] & 0xFFFFu);
       c[2 * q + 1] = ecc_correction<true, true>(x[2 * q + 1], pk >> 16, rnd.w[q] >> 16);
     }
-    cw[0] = pack_bytes(c[0], c[1], c[2], c[3]);
-    cw[1] = pack_bytes(c[4], c[5], c[6], c[7]);
+    if constexpr (E == 2) {
+      cw[0] = __builtin_amdgcn_perm((uint32_t)c[1], (uint32_t)c[0], 0x0c0c0400u);
+    } else {
+#pragma unroll
+      for (int q = 0; q < E / 4; ++q) cw[q] = pack_bytes(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]);
+    }
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < E; ++j) {
       uint32_t h;
       if (F == HB_FMT_BF16) {
         h = sr_bf16(x[j], rnd.bits16(j));
@@ -259,24 +385,22 @@ __device__ __forceinline__ void raw_encode_s(Raw& r, const float (&x)[8], const 
       w[j >> 1] |= (h & 0xFFFFu) << ((j & 1) * 16);
     }
   }
-  r.a = make_uint4(w[0], w[1], w[2], w[3]);
-  r.c = make_uint4(cw[0], cw[1], cw[2], cw[3]);
+#pragma unroll
+  for (int i = 0; i < E / 2; ++i) {
+    r.a[i] = w[i];
+    r.c[i] = cw[i];
+  }
 }
 
-template <int F>
-__device__ __forceinline__ void raw_store_s(const Raw& r, char* prim, char* corr, int64_t idx) {
+template <int F, int E>
+__device__ __forceinline__ void raw_store_s(const RawT<E>& r, char* prim, char* corr, int64_t idx) {
   if (F == HB_FMT_F32) {
-    uint4* p = reinterpret_cast<uint4*>(prim + idx * 4);
-    p[0] = r.a;
-    p[1] = r.b;
+    st_slab<4 * E>(prim + idx * 4, r.a);
   } else {
-    *reinterpret_cast<uint4*>(prim + idx * 2) = r.a;
+    st_slab<2 * E>(prim + idx * 2, r.a);
     if (fmt_is_ecc(F)) {
-      if (fmt_corr8(F)) {
-        *reinterpret_cast<uint2*>(corr + idx) = make_uint2(r.c.x, r.c.y);
-      } else {
-        *reinterpret_cast<uint4*>(corr + idx * 2) = r.c;
-      }
+      if (fmt_corr8(F)) st_slab<E>(corr + idx, r.c);
+      else st_slab<2 * E>(corr + idx * 2, r.c);
     }
   }
 }
@@ -299,29 +423,34 @@ __device__ __forceinline__ void raw_store_s(const Raw& r, char* prim, char* corr
     }                                                             \
   } while (0)
 
-template <int F>
-__device__ __forceinline__ void raw_load(Raw& r, int f, const char* prim, const char* corr, int64_t idx) {
-#define HB_CALL(X) raw_load_s<X>(r, prim, corr, idx)
+template <int F, int E>
+__device__ __forceinline__ void raw_load(RawT<E>& r, int f, const char* prim, const char* corr, int64_t idx) {
+#define HB_CALL(X) raw_load_s<X, E>(r, prim, corr, idx)
   HB_FMT_SWITCH(F, f, HB_CALL);
 #undef HB_CALL
 }
-template <int F>
-__device__ __forceinline__ void raw_decode(const Raw& r, int f, float (&x)[8]) {
-#define HB_CALL(X) raw_decode_s<X>(r, x)
+template <int F, int E>
+__device__ __forceinline__ void raw_decode(const RawT<E>& r, int f, float (&x)[E]) {
+#define HB_CALL(X) raw_decode_s<X, E>(r, x)
   HB_FMT_SWITCH(F, f, HB_CALL);
 #undef HB_CALL
 }
+template <int F, int E>
+__device__ __forceinline__ void raw_encode(RawT<E>& r, int f, const float (&x)[E], const Noise<E>& rnd) {
+#define HB_CALL(X) raw_encode_s<X, E>(r, x, rnd)
+  HB_FMT_SWITCH(F, f, HB_CALL);
+#undef HB_CALL
+}
+template <int F, int E>
+__device__ __forceinline__ void raw_store(const RawT<E>& r, int f, char* prim, char* corr, int64_t idx) {
+#define HB_CALL(X) raw_store_s<X, E>(r, prim, corr, idx)
+  HB_FMT_SWITCH(F, f, HB_CALL);
+#undef HB_CALL
+}
+// octet kernels hand their noise over as the four words of a Rand8
 template <int F>
 __device__ __forceinline__ void raw_encode(Raw& r, int f, const float (&x)[8], const Rand8& rnd) {
-#define HB_CALL(X) raw_encode_s<X>(r, x, rnd)
-  HB_FMT_SWITCH(F, f, HB_CALL);
-#undef HB_CALL
-}
-template <int F>
-__device__ __forceinline__ void raw_store(const Raw& r, int f, char* prim, char* corr, int64_t idx) {
-#define HB_CALL(X) raw_store_s<X>(r, prim, corr, idx)
-  HB_FMT_SWITCH(F, f, HB_CALL);
-#undef HB_CALL
+  raw_encode<F, 8>(r, f, x, Noise<8>{{rnd.w[0], rnd.w[1], rnd.w[2], rnd.w[3]}});
 }
 
 // element-wise (tail) access to a plain gradient buffer that is NOT slab-padded
@@ -352,6 +481,14 @@ __device__ __forceinline__ float sqrt_rn_normal(float x) {
   s = r_lo <= 0.0f ? lo : s;
   s = r_hi > 0.0f ? hi : s;
   return s;
+}
+
+// fmaxf(x, lo) for an x that is never a signalling NaN (the result of a square root) and a lo that is a number: the
+// hardware maximum returns the operand that is not a NaN, as fmaxf does; the builtin would first canonicalise both.
+__device__ __forceinline__ float max_nonnan(float x, float lo) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(lo));
+  return r;
 }
 
 // ---------------------------------------------------------------------------------------------------------

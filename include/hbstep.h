@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 5
+#define HB_ABI_VERSION 6
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -76,10 +76,12 @@ enum {
 /* where the noise of stochastic rounding comes from */
 enum {
   HB_RNG_HALF = 0,   /* uniform = 0.5, 16-bit noise = 0x8000: deterministic ("rounding disabled") */
-  HB_RNG_PHILOX = 1, /* Philox4x32-10, counter (flat_index >> 3, step, stream), key = seed */
+  HB_RNG_PHILOX = 1, /* Philox4x32-10, counter (flat_index >> 2, step, stream >> 1), key = seed: one call serves 4 consecutive
+                      * elements for the streams 2p and 2p + 1; element j of stream s takes the 16 bits at half-word j of the
+                      * words (s & 1) * 2 and (s & 1) * 2 + 1 */
 };
 
-/* Philox stream ids: one per rounding site of the step */
+/* Philox stream ids: one per rounding site of the step (exp_avg and exp_avg_sq share their calls) */
 enum {
   HB_STREAM_MARS_SR = 0,
   HB_STREAM_OLD_GRAD = 1,
@@ -174,7 +176,7 @@ int hb_ecc_encode(const float* src, void* primary, void* corr, int64_t n, int32_
 int hb_ecc_decode(const void* primary, const void* corr, float* dst, int64_t n, int32_t fmt, void* stream);
 int hb_sr_bf16(const float* src, void* dst_bf16, int64_t n, int32_t rng_mode, uint64_t seed, uint32_t step,
                uint32_t stream_id, int64_t flat_base, void* stream);
-/* raw Philox words for n octets starting at octet q0: out[4*n] */
+/* raw Philox words of n calls with counters (q, step, stream_id), q = q0 .. q0 + n - 1: out[4*n] */
 int hb_philox_words(uint32_t* out, int64_t n, uint64_t q0, uint64_t seed, uint32_t step, uint32_t stream_id, void* stream);
 
 /* per-tensor sum of squares over a slab role, the reduction behind the clipping norms

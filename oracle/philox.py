@@ -8,10 +8,15 @@ easy as 1, 2, 3" (SC'11), Philox4x32 with 10 rounds, keyed so that any element's
 noise is a pure function of (seed, step, stream, flat element index).  This file
 is the CPU statement of that layout:
 
-    octet   q = flat_index >> 3            (8 consecutive elements share one call)
-    counter = (q & 0xffffffff, q >> 32, step & 0xffffffff, stream)
+    quartet q = flat_index >> 2            (4 consecutive elements, for the two streams 2p and 2p + 1 of a
+                                            stream pair p, share one call)
+    counter = (q & 0xffffffff, q >> 32, step & 0xffffffff, stream >> 1)
     key     = (seed & 0xffffffff, seed >> 32)
-    element j = flat_index & 7 takes 16 bits: word j >> 1, low half if j even else high half
+    element j = flat_index & 3 of stream s takes 16 bits: word (s & 1) * 2 + (j >> 1), low half if j even else
+    high half
+
+exp_avg (stream 2) and exp_avg_sq (stream 3) form a pair, so a lane that owns a quartet of the slab makes one call
+for both moments.
 
 Known-answer vectors from the Random123 distribution (kat_vectors) are checked
 in tests/test_oracle_philox.py.
@@ -61,17 +66,18 @@ def bits16(seed: int, step: int, stream: int, flat_index) -> np.ndarray:
     index inside the tensor), any integer array.
     """
     f = np.asarray(flat_index, dtype=np.uint64)
-    q = f >> np.uint64(3)
-    j = (f & np.uint64(7)).astype(np.int64)
+    q = f >> np.uint64(2)
+    j = (f & np.uint64(3)).astype(np.int64)
+    stream = int(stream) & 0xFFFFFFFF
     out = philox4x32_10(
         q & _MASK,
         q >> _S32,
         np.full_like(q, int(step) & 0xFFFFFFFF),
-        np.full_like(q, int(stream) & 0xFFFFFFFF),
+        np.full_like(q, stream >> 1),
         int(seed) & 0xFFFFFFFF,
         (int(seed) >> 32) & 0xFFFFFFFF,
     )
     words = np.stack(out, axis=-1)  # [..., 4]
-    w = np.take_along_axis(words, (j >> 1)[..., None].astype(np.int64), axis=-1)[..., 0]
+    w = np.take_along_axis(words, ((stream & 1) * 2 + (j >> 1))[..., None].astype(np.int64), axis=-1)[..., 0]
     shift = ((j & 1) * 16).astype(np.uint64)
     return ((w >> shift) & np.uint64(0xFFFF)).astype(np.int64)

@@ -27,19 +27,20 @@ def test_philox_known_answers():
 
 
 def test_philox_layout():
-    """eight consecutive elements share one call; element j takes half-word j of the 128-bit block."""
-    seed, step, stream = 0x1234_5678_9ABC_DEF0, 7, 3
-    idx = np.arange(8 * 5, 8 * 5 + 8)
-    bits = philox.bits16(seed, step, stream, idx)
-    w = philox.philox4x32_10(5, 0, step, stream, seed & 0xFFFFFFFF, seed >> 32)
-    want = []
-    for word in w:
-        want += [int(word) & 0xFFFF, int(word) >> 16]
-    assert bits.tolist() == want
+    """four consecutive elements and the two streams of a pair share one call: stream 2p takes words 0 and 1, stream
+    2p + 1 words 2 and 3; element j takes half-word j of its stream's two words."""
+    seed, step = 0x1234_5678_9ABC_DEF0, 7
+    idx = np.arange(4 * 5, 4 * 5 + 4)
+    w = [int(x) for x in philox.philox4x32_10(5, 0, step, 1, seed & 0xFFFFFFFF, seed >> 32)]
+    assert philox.bits16(seed, step, 2, idx).tolist() == [w[0] & 0xFFFF, w[0] >> 16, w[1] & 0xFFFF, w[1] >> 16]
+    assert philox.bits16(seed, step, 3, idx).tolist() == [w[2] & 0xFFFF, w[2] >> 16, w[3] & 0xFFFF, w[3] >> 16]
+    # another pair is another counter word, not another half of the same call
+    w4 = [int(x) for x in philox.philox4x32_10(5, 0, step, 2, seed & 0xFFFFFFFF, seed >> 32)]
+    assert philox.bits16(seed, step, 4, idx).tolist() == [w4[0] & 0xFFFF, w4[0] >> 16, w4[1] & 0xFFFF, w4[1] >> 16]
     # high counter word
-    big = np.array([(1 << 35) + 3], dtype=np.uint64)
-    w = philox.philox4x32_10(0, 1, step, stream, seed & 0xFFFFFFFF, seed >> 32)
-    assert philox.bits16(seed, step, stream, big)[0] == (int(w[1]) >> 16)
+    big = np.array([(1 << 34) + 3], dtype=np.uint64)
+    w = philox.philox4x32_10(0, 1, step, 1, seed & 0xFFFFFFFF, seed >> 32)
+    assert philox.bits16(seed, step, 3, big)[0] == (int(w[3]) >> 16)
 
 
 @pytest.mark.parametrize("mode", list(ecc.MODES))
