@@ -9,7 +9,8 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_uint32, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libhbstep.so")
+# HBSTEP_LIB names another build of the library (same ABI), e.g. one compiled with different tuning constants
+LIB_PATH = os.environ.get("HBSTEP_LIB") or os.path.join(_HERE, "libhbstep.so")
 
 # include/hbstep.h
 ABI_VERSION = 6  # HB_ABI_VERSION this binding was written against
@@ -17,7 +18,7 @@ FMT_F32, FMT_BF16, FMT_F16, FMT_ECC_BF16_8, FMT_ECC_BF16_16, FMT_ECC_F16_8, FMT_
 ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD = 1, 2, 4, 8, 16, 32, 64
 RNG_HALF, RNG_PHILOX = 0, 1
-STREAM_MARS_SR, STREAM_OLD_GRAD, STREAM_EXP_AVG, STREAM_EXP_AVG_SQ, STREAM_PARAM, STREAM_INIT_PARAM, STREAM_NS_INPUT = range(7)
+STREAM_MARS_SR, STREAM_PARAM, STREAM_EXP_AVG, STREAM_EXP_AVG_SQ, STREAM_OLD_GRAD, STREAM_INIT_PARAM, STREAM_NS_INPUT = range(7)
 STREAM_CLIP, STREAM_EXP_AVG_SLOW = 8, 9
 NS_LEGACY, NS_BF16_UPDATE = 1, 2
 NOALLOC_MAX_TENSORS = 65536  # HB_NOALLOC_MAX_TENSORS

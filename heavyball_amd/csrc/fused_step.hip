@@ -210,16 +210,22 @@ namespace hb {
 static int run_fused_step(const HbStepDesc* d, StepArgs& a, uint32_t* counts, hipStream_t stream, const char* what) {
   const bool mars = (d->flags & HB_FLAG_MARS) != 0;
   const bool caution = (d->flags & HB_FLAG_CAUTION) != 0;
-  const int grid = persistent_grid(d->n_chunks * kSub);
-  if (grid <= 0) return set_error(HB_ELAUNCH, "could not query the device");
   a.counts = counts;
+  auto launch = [&](int pass) {
+    const StepKernel k = pick_kernel(d->algo, mars, pass, a.pf, a.gf, a.sf);
+    const int grid = persistent_grid(d->n_chunks * k.sub);
+    if (grid <= 0) return false;
+    k.fn<<<grid, kThreads, 0, stream>>>(a);
+    return true;
+  };
+  bool ok;
   if (caution) {
     zero_u32_kernel<<<(d->n_tensors + 255) / 256, 256, 0, stream>>>(counts, d->n_tensors);
-    pick_kernel(d->algo, mars, kCautionCount, a.pf, a.gf, a.sf)<<<grid, kThreads, 0, stream>>>(a);
-    pick_kernel(d->algo, mars, kCautionApply, a.pf, a.gf, a.sf)<<<grid, kThreads, 0, stream>>>(a);
+    ok = launch(kCautionCount) && launch(kCautionApply);
   } else {
-    pick_kernel(d->algo, mars, kNoCaution, a.pf, a.gf, a.sf)<<<grid, kThreads, 0, stream>>>(a);
+    ok = launch(kNoCaution);
   }
+  if (!ok) return set_error(HB_ELAUNCH, "could not query the device");
   return check_launch(what);
 }
 

@@ -9,28 +9,30 @@
 
 namespace hb {
 
-// Work decomposition of the step kernel: every lane owns HB_EPL consecutive elements of each role per group, a workgroup
-// of HB_THREADS lanes takes kWork = HB_THREADS * HB_EPL * HB_GROUPS consecutive elements, and a chunk of the chunk table
-// is kSub such work units.  Measured on MI355X: the narrower the run of a lane, the closer the kernel gets to the
-// bandwidth of a plain copy (an arithmetic-free kernel with the access pattern of the ECC LaProp step moves 5.8 TB/s with
-// 8 elements per lane, 6.0 with 4, 6.3 with 2), and one group per lane beats two (all loads of a wavefront are in flight
-// at once with few registers, so more wavefronts fit and reads and writes alternate at a finer grain).
+// Work decomposition of the step kernel: every lane owns E consecutive elements of each role per group, a workgroup of
+// kThreads lanes takes kWork = kThreads * E * G consecutive elements (G groups per lane, all loads issued before any
+// arithmetic), and a chunk of the chunk table is kSub such work units.  Measured on MI355X over E = 2, 4, 8, G = 1, 2, 4
+// and 64 ... 512 lanes: the pass that reads and writes every role is fastest with narrow runs (an arithmetic-free kernel
+// with the access pattern of the ECC LaProp step moves 5.8 TB/s with 8 elements per lane, 6.0 with 4, 6.3 with 2; the real
+// kernel turns compute-bound at 2), the read-only count pass of caution with wide ones.
 #ifndef HB_THREADS
 #define HB_THREADS 256
 #endif
-#ifndef HB_GROUPS
-#define HB_GROUPS 1
-#endif
-#ifndef HB_EPL
-#define HB_EPL 4
-#endif
 constexpr int kThreads = HB_THREADS;
-constexpr int kGroups = HB_GROUPS;
-constexpr int kE = HB_EPL;
-constexpr int kWork = kThreads * kE * kGroups;
-constexpr int kSub = HB_CHUNK / kWork;
-static_assert(kE == 2 || kE == 4 || kE == 8, "2, 4 or 8 elements per lane");
-static_assert(kSub >= 1 && kSub * kWork == HB_CHUNK, "a chunk must be a whole number of work units");
+template <int E_, int G_>
+struct Geo {
+  static constexpr int E = E_, G = G_;
+  static constexpr int kWork = kThreads * E * G;
+  static constexpr int kSub = HB_CHUNK / kWork;
+  static_assert(E == 2 || E == 4 || E == 8, "2, 4 or 8 elements per lane");
+  static_assert(kSub >= 1 && kSub * kWork == HB_CHUNK, "a chunk must be a whole number of work units");
+};
+#ifndef HB_GEO_STEP
+#define HB_GEO_STEP Geo<4, 2>
+#endif
+#ifndef HB_GEO_COUNT
+#define HB_GEO_COUNT Geo<8, 2>
+#endif
 
 struct StepArgs {
   char* param;
@@ -67,10 +69,11 @@ __device__ __forceinline__ void for_each_index(F&& f, std::integer_sequence<int,
 }
 
 // One work unit.  FULL = every lane's elements are inside the tensor (the common case): no bounds tests at all.
-template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF, bool FULL>
+template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF, bool FULL, class GEO>
 __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, const int gf, const int sf, const int t, const int valid,
                                            const int64_t flat0, const char* gbase, const int64_t g0, const bool g_slab, const float scale,
                                            const float gw, const float ew) {
+  constexpr int kE = GEO::E, kGroups = GEO::G;
   constexpr bool kCount = CAUTION == kCautionCount;
   constexpr bool kAdopt = ALGO == HB_ALGO_ADOPT, kMix = ALGO == HB_ALGO_ADEMAMIX, kNadam = ALGO == HB_ALGO_NADAM;
   // the count pass of Adam and AdEMAMix needs only the sign of the numerator of the update
@@ -91,8 +94,9 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   RawT<kE> rp[kGroups], rg[kGroups], rm[kGroups], rv[kGroups], ro[kGroups], rs[kGroups];
   float gtail[kGroups][kE];
   bool tail[kGroups];
-#pragma unroll
-  for (int k = 0; k < kGroups; ++k) {
+  // the loads of one group
+  auto fetch = [&](auto kc) {
+    constexpr int k = decltype(kc)::value;
     const int e = k * (kThreads * kE) + threadIdx.x * kE;
     tail[k] = false;
     if (FULL || e < valid) {
@@ -111,7 +115,8 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
       if (MARS) raw_load<SF>(ro[k], sf, a.og, a.og_corr, idx);
       if ((!kCount && (!kAdopt || !warmup)) || (kNadam && coupled)) raw_load<PF>(rp[k], pf, a.param, a.param_corr, idx);
     }
-  }
+  };
+  for_each_index(fetch, std::make_integer_sequence<int, kGroups>{});
 
   uint32_t masked = 0;
   // One group.  A generic lambda over a compile-time index instead of an unrolled loop: with run-time format codes
@@ -122,6 +127,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
     if (!FULL && e >= valid) return;
     const int64_t idx = flat0 + e;
     float p[kE], g[kE], m[kE], v[kE], og[kE], u[kE], sl[kE];
+    Noise<kE> rn_p{};  // noise of the parameter's rounding
     if (!FULL && tail[k]) {
 #pragma unroll
       for (int j = 0; j < kE; ++j) g[j] = gtail[k][j];
@@ -135,8 +141,9 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
 
     if (MARS) {
       raw_decode<SF>(ro[k], sf, og);
-      Noise<kE> rn{}, rn_og{};  // streams HB_STREAM_MARS_SR and HB_STREAM_OLD_GRAD share their Philox calls
-      if (gf == HB_FMT_BF16 || (og_rounds && !kCount)) a.rng.noise_pair<kE>(idx, HB_STREAM_MARS_SR >> 1, rn, rn_og);
+      Noise<kE> rn{};  // HB_STREAM_MARS_SR shares its Philox calls with HB_STREAM_PARAM (rn_p, used at the end)
+      if (gf == HB_FMT_BF16) a.rng.noise_pair<kE>(idx, HB_STREAM_MARS_SR >> 1, rn, rn_p);
+      else if (pf != HB_FMT_F32 && !kCount) rn_p = a.rng.noise<kE>(idx, HB_STREAM_PARAM);
 #pragma unroll
       for (int j = 0; j < kE; ++j) {
         float gc = g[j] * a.omamars + og[j] * a.amars;  // heavyball/utils.py:1048
@@ -147,7 +154,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
       }
       if (!kCount) {
         RawT<kE> w;
-        if (!og_rounds) rn_og = Noise<kE>{};
+        const Noise<kE> rn_og = og_rounds ? a.rng.noise<kE>(idx, HB_STREAM_OLD_GRAD) : Noise<kE>{};
         raw_encode<SF>(w, sf, og, rn_og);
         raw_store<SF>(w, sf, a.og, a.og_corr, idx);
         if (write_grad) {
@@ -235,8 +242,8 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
         raw_store<SF>(w, sf, a.s3, a.s3_corr, idx);
       }
       if (!kAdopt || !warmup) {
-        const Noise<kE> rn = pf != HB_FMT_F32 ? a.rng.noise<kE>(idx, HB_STREAM_PARAM) : Noise<kE>{};
-        raw_encode<PF>(w, pf, p, rn);
+        if (!MARS && pf != HB_FMT_F32) rn_p = a.rng.noise<kE>(idx, HB_STREAM_PARAM);
+        raw_encode<PF>(w, pf, p, rn_p);
         raw_store<PF>(w, pf, a.param, a.param_corr, idx);
       }
     }
@@ -249,8 +256,9 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   }
 }
 
-template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF>
+template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF, class GEO>
 __global__ __launch_bounds__(kThreads) void fused_step_kernel(const StepArgs a) {
+  constexpr int kWork = GEO::kWork, kSub = GEO::kSub;
   const int pf = PF == kDyn ? a.pf : PF;
   const int gf = GF == kDyn ? a.gf : GF;
   const int sf = SF == kDyn ? a.sf : SF;
@@ -278,23 +286,29 @@ __global__ __launch_bounds__(kThreads) void fused_step_kernel(const StepArgs a) 
       gw = a.tscal[2 * t];
       ew = a.tscal[2 * t + 1];
     }
-    if (valid == kWork) step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, true>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
-    else step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, false>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
+    if (valid == kWork) step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, true, GEO>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
+    else step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, false, GEO>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
   }
 }
 
-using StepKernel = void (*)(const StepArgs);
+// a kernel and the number of its work units per chunk (the grid is n_chunks * sub workgroups)
+struct StepKernel {
+  void (*fn)(const StepArgs);
+  int sub;
+};
 
 template <int ALGO, int PF, int GF, int SF>
 inline StepKernel pick_pass(bool mars, int caution) {
+  using S = HB_GEO_STEP;
+  using C = HB_GEO_COUNT;
   if (mars) {
-    if (caution == kNoCaution) return fused_step_kernel<ALGO, true, kNoCaution, PF, GF, SF>;
-    if (caution == kCautionCount) return fused_step_kernel<ALGO, true, kCautionCount, PF, GF, SF>;
-    return fused_step_kernel<ALGO, true, kCautionApply, PF, GF, SF>;
+    if (caution == kNoCaution) return {fused_step_kernel<ALGO, true, kNoCaution, PF, GF, SF, S>, S::kSub};
+    if (caution == kCautionCount) return {fused_step_kernel<ALGO, true, kCautionCount, PF, GF, SF, C>, C::kSub};
+    return {fused_step_kernel<ALGO, true, kCautionApply, PF, GF, SF, S>, S::kSub};
   }
-  if (caution == kNoCaution) return fused_step_kernel<ALGO, false, kNoCaution, PF, GF, SF>;
-  if (caution == kCautionCount) return fused_step_kernel<ALGO, false, kCautionCount, PF, GF, SF>;
-  return fused_step_kernel<ALGO, false, kCautionApply, PF, GF, SF>;
+  if (caution == kNoCaution) return {fused_step_kernel<ALGO, false, kNoCaution, PF, GF, SF, S>, S::kSub};
+  if (caution == kCautionCount) return {fused_step_kernel<ALGO, false, kCautionCount, PF, GF, SF, C>, C::kSub};
+  return {fused_step_kernel<ALGO, false, kCautionApply, PF, GF, SF, S>, S::kSub};
 }
 
 // The kernel of one algorithm for a (param, grad, state) format triple: three triples are statically specialised,

@@ -84,10 +84,10 @@ enum {
 /* Philox stream ids: one per rounding site of the step (exp_avg and exp_avg_sq share their calls) */
 enum {
   HB_STREAM_MARS_SR = 0,
-  HB_STREAM_OLD_GRAD = 1,
+  HB_STREAM_PARAM = 1, /* pairs with HB_STREAM_MARS_SR: a step with MARS and a narrow parameter makes one call for both */
   HB_STREAM_EXP_AVG = 2,
   HB_STREAM_EXP_AVG_SQ = 3,
-  HB_STREAM_PARAM = 4,
+  HB_STREAM_OLD_GRAD = 4,
   HB_STREAM_INIT_PARAM = 5,
   HB_STREAM_NS_INPUT = 6, /* the legacy Newton-Schulz variant also draws from 7 for its second rounding */
   HB_STREAM_CLIP = 8,     /* bf16 stochastic rounding of a clipped bf16 gradient */

@@ -33,10 +33,10 @@ _S32 = np.uint64(32)
 
 # stream ids: which rounding site inside the step consumes the numbers
 STREAM_MARS_SR = 0  # bf16 stochastic rounding of the MARS-corrected gradient
-STREAM_OLD_GRAD = 1  # ECC / SR write of mars_old_grad
+STREAM_PARAM = 1  # ECC / SR write of the parameter (shares its calls with STREAM_MARS_SR)
 STREAM_EXP_AVG = 2  # ECC / SR write of exp_avg
-STREAM_EXP_AVG_SQ = 3  # ECC / SR write of exp_avg_sq
-STREAM_PARAM = 4  # ECC / SR write of the parameter
+STREAM_EXP_AVG_SQ = 3  # ECC / SR write of exp_avg_sq (shares its calls with STREAM_EXP_AVG)
+STREAM_OLD_GRAD = 4  # ECC / SR write of mars_old_grad
 STREAM_INIT_PARAM = 5  # param::ecc initial correction at construction
 STREAM_NS_INPUT = 6  # bf16 stochastic rounding of the Newton-Schulz input (the legacy variant also uses 7)
 STREAM_CLIP = 8  # bf16 stochastic rounding of a clipped bf16 gradient
