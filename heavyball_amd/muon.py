@@ -137,6 +137,7 @@ class Muon(HBOptimizer):
         for b, items in per_bucket.values():
             if b.device.type != "cuda":
                 raise _lib.HbError("the optimizer step runs on the GPU only: parameters must live on a CUDA/HIP device")
+            self._check_home(b, items)
             b.slab.role(self.KEY, mom_prim)
             if mom_corr is not None:
                 b.slab.role(self.KEY + "::ecc", mom_corr)
@@ -170,6 +171,7 @@ class Muon(HBOptimizer):
         if self.update_clipping is not None and any(g.dtype != torch.float32 for _, g in active) and not self.promote:
             raise NotImplementedError("update_clipping with 16-bit gradients (the reference rounds the clipped update to their dtype)")
         keep = []
+        tables = {}  # (bucket, gradient dtype) -> device table of gradient pointers
         for b, items, by_dtype in prepared:
             offsets, numel = b.slab.meta()
             stream = current_stream_ptr(b.device)
@@ -181,7 +183,7 @@ class Muon(HBOptimizer):
                     ptrs = [0] * len(b.params)
                     for i, g in lst:
                         ptrs[i] = g.data_ptr()
-                    table = b.grad_ptr_table(gdt, ptrs)  # the raw gradients: caution compares the update against them
+                    table = tables[(id(b), gdt)] = b.grad_ptr_table(gdt, ptrs)  # the raw gradients: caution compares the update against them
                     if clip is None:
                         g_slab, g_table, g_fmt = None, table.data_ptr(), _PLAIN_FMT[gdt]
                     else:  # the clipped gradients live in a slab role
@@ -233,7 +235,7 @@ class Muon(HBOptimizer):
                 for gdt, lst in by_dtype.items():
                     act = tuple(i for i, _ in lst)
                     chunks, n_chunks = b.slab.chunks(act)
-                    table = b.grad_tables[gdt][0]
+                    table = tables[(id(b), gdt)]
                     d = _lib.HbStepDesc()
                     d.param, d.param_corr = b.slab.ptr("param"), b.slab.ptr("param::ecc")
                     d.grad, d.grad_ptrs = None, table.data_ptr()

@@ -130,7 +130,9 @@ class Bucket:
         self.param_dtype = param_dtype
         self.slab = Slab([p.shape for p in params], self.device)
         self.counts = None  # caution scratch
-        self.grad_tables: Dict[Tuple, Tuple[torch.Tensor, tuple]] = {}
+        self.grad_tables: Dict[Tuple, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self._home = None
+        self.state_ready = {}  # state layout key -> indices of the tensors whose state entries exist
 
     def caution_scratch(self) -> torch.Tensor:
         if self.counts is None:
@@ -138,17 +140,28 @@ class Bucket:
         return self.counts
 
     def grad_ptr_table(self, key, ptrs: List[int]) -> torch.Tensor:
-        """Device array of per-tensor gradient pointers (indexed by slab tensor index); re-uploaded only on change."""
-        hit = self.grad_tables.get(key)
-        tup = tuple(ptrs)
-        if hit is not None and hit[1] == tup:
+        """Device array of per-tensor gradient pointers (indexed by slab tensor index).  Gradient buffers usually come back
+        at the addresses of a few steps ago (the caching allocator, or a handful of buffers in rotation), so the last
+        few tables are kept and one is uploaded only for a set of pointers not seen among them."""
+        tup = (key, *ptrs)
+        hit = self.grad_tables.get(tup)
+        if hit is not None:
             return hit[0]
         host = torch.tensor(ptrs, dtype=torch.int64)
         if self.device.type == "cuda":
             host = host.pin_memory()
         dev = host.to(self.device, non_blocking=True)
-        self.grad_tables[key] = (dev, tup, host)
+        if len(self.grad_tables) >= 16:
+            self.grad_tables.pop(next(iter(self.grad_tables)))  # oldest first; a kernel in flight keeps its table through _last_launch
+        self.grad_tables[tup] = (dev, host)
         return dev
+
+    def home_ptrs(self) -> List[int]:
+        """Address of every parameter's view of the slab: what ``p.data_ptr()`` must be while the slab backs ``p``."""
+        if self._home is None:
+            base, size = self.slab.ptr("param"), self.slab.roles["param"].element_size()
+            self._home = [base + int(o) * size for o in self.slab.offsets_np]
+        return self._home
 
 
 class HBOptimizer(torch.optim.Optimizer):
@@ -196,6 +209,7 @@ class HBOptimizer(torch.optim.Optimizer):
         base.update({k: v for k, v in defaults.items() if v is not use_default})
         base.setdefault("multi_tensor", True)
         self._buckets: Dict[int, List[Bucket]] = {}
+        self._loc: Dict[int, Tuple[Bucket, int]] = {}  # id(parameter) -> (bucket, index in the bucket)
         self.rng_seed = int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF
         self.use_ema = False
         self.inner_group = {}
@@ -258,6 +272,8 @@ class HBOptimizer(torch.optim.Optimizer):
                 if pecc:
                     self._state0(p)["param::ecc"] = b.slab.view("param::ecc", i)
             buckets.append(b)
+            for i, p in enumerate(plist):
+                self._loc[id(p)] = (b, i)
         self._buckets[gi] = buckets
 
     def _route(self, p) -> int:
@@ -309,11 +325,28 @@ class HBOptimizer(torch.optim.Optimizer):
         return total
 
     def _find_bucket(self, gi: int, p) -> Tuple[Bucket, int]:
-        for b in self._buckets[gi]:
-            i = b.index.get(id(p))
-            if i is not None:
-                return b, i
-        raise KeyError("Tensor has no tracked state.")
+        loc = self._loc.get(id(p))
+        if loc is None or loc[0].params[loc[1]] is not p:
+            raise KeyError("Tensor has no tracked state.")
+        return loc
+
+    def _check_home(self, b: Bucket, items):
+        """``step()`` updates the slab, so ``p.data`` must still be the slab's view of ``p``.  A parameter whose data was
+        rebound since (``model.bfloat16()``, ``p.data = ...``, a swap of averaged weights) is moved back: its current
+        values are copied into the slab and ``p.data`` is pointed there again, as after ``load_state_dict``.
+        ``items``: [(index, parameter, ...)]."""
+        home = b.home_ptrs()
+        for it in items:
+            i, p = it[0], it[1]
+            if p.data_ptr() != home[i] and p.numel():
+                view = b.slab.view("param", i)
+                if p.device != b.device:
+                    raise _lib.HbError("a parameter was moved to another device after the optimizer was constructed")
+                if p.dtype != view.dtype:
+                    raise _lib.HbError(f"a parameter changed its dtype from {view.dtype} to {p.dtype} after the optimizer was constructed; "
+                                       "construct the optimizer after casting the model")  # fmt: skip
+                view.copy_(p.data)
+                p.data = view
 
     # -- step ----------------------------------------------------------------------------------------------------
     def _schedule_tick(self):
@@ -364,7 +397,7 @@ class HBOptimizer(torch.optim.Optimizer):
                 continue
             if self.consume_grad:
                 p.grad = None
-            active.append((p, g.detach()))
+            active.append((p, g))
         if not active:
             return
         step = group.get("_group_step")
@@ -513,6 +546,7 @@ class HBOptimizer(torch.optim.Optimizer):
             if gi not in self._buckets:
                 self._adopt_group(gi, group)
             for b in self._buckets[gi]:
+                b.state_ready.clear()
                 for i, p in enumerate(b.params):
                     if p not in self.state:
                         continue
@@ -580,6 +614,11 @@ class FirstOrder(HBOptimizer):
         _, prim, corr = self._state_fmt(group)
         mars = group.get("mars", False)
         names = list(self._moment_keys(group).values()) + ([k_o] if mars else [])
+        ready = b.state_ready.setdefault((tuple(names), prim, corr), set())
+        if len(ready) == len(b.params) or ready.issuperset(idx):
+            if names[0] in self.state[b.params[idx[0]]].get(0, ()):
+                return
+            ready.clear()  # optimizer.state was emptied by the caller: build the entries again
         for k in names:
             b.slab.role(k, prim)
             if corr is not None:
@@ -594,6 +633,7 @@ class FirstOrder(HBOptimizer):
                 if corr is not None:
                     st.setdefault(k + "::ecc", b.slab.view(k + "::ecc", i))
             st.setdefault("is_initialized", set()).update(init_ids)
+        ready.update(idx)
 
     def _betas(self, group, step):
         beta1 = group["betas"][0] if group.get("beta") is None else group["beta"]
@@ -671,20 +711,24 @@ class FirstOrder(HBOptimizer):
         for b, items in per_bucket.values():
             if b.device.type != "cuda":
                 raise _lib.HbError("the optimizer step runs on the GPU only: parameters must live on a CUDA/HIP device")
+            self._check_home(b, items)
             self._ensure_state(group, b, [i for i, _, _ in items])
             by_dtype: Dict[torch.dtype, List] = {}
+            f32_t, promote = torch.float32, self.promote
             for i, p, g in items:
                 if g.is_sparse:
                     raise NotImplementedError("sparse gradients")
-                if self.promote and g.dtype != torch.float32:
-                    g = g.float()
-                if g.dtype not in _PLAIN_FMT:
-                    g = g.float()
+                dt = g.dtype
+                if dt is not f32_t and (promote or dt not in _PLAIN_FMT):
+                    g, dt = g.float(), f32_t
                 if g.shape != p.shape:
                     raise ValueError(f"gradient shape {tuple(g.shape)} does not match parameter shape {tuple(p.shape)}")
-                if not g.is_contiguous() or g.data_ptr() % 16 or g.device != b.device:
-                    g = g.to(b.device).clone(memory_format=torch.contiguous_format)
-                by_dtype.setdefault(g.dtype, []).append((i, g))
+                if g.data_ptr() & 15 or not g.is_contiguous() or g.device != b.device:
+                    g = g.detach().to(b.device).clone(memory_format=torch.contiguous_format)
+                lst = by_dtype.get(dt)
+                if lst is None:
+                    lst = by_dtype[dt] = []
+                lst.append((i, g))
             if self.gradient_clipping is not None and len(by_dtype) > 1:
                 raise NotImplementedError("gradient_clipping with gradients of several dtypes in one bucket")
             for gdt, lst in by_dtype.items():

@@ -159,6 +159,7 @@ class SOAP(HBOptimizer):
         for key, (b, items) in per_bucket.items():
             if b.device.type != "cuda":
                 raise _lib.HbError("the optimizer step runs on the GPU only: parameters must live on a CUDA/HIP device")
+            self._check_home(b, items)
             if b.param_dtype != torch.float32:
                 raise NotImplementedError("SOAP on the HIP kernels takes fp32 parameters")
             if any(g.dtype != torch.float32 for _, _, g in items) and not self.promote:

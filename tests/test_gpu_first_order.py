@@ -356,3 +356,31 @@ def test_state_dict_layout_matches_reference(case):
     torch.save(sd, buf)
     buf.seek(0)
     torch.load(buf, weights_only=True)
+
+
+def test_parameter_rebound_after_construction_is_moved_back_into_the_slab():
+    """``p.data`` pointed at fresh storage after the optimizer was built (a swap of averaged weights, ``p.data = ...``):
+    the next step must act on the new values and leave the result in ``p``, not in an orphaned slab copy."""
+    shapes = [(64, 96), (96,), (1000, 33)]
+    host, params, opt, orc = H.build_pair(heavyball_amd.AdamW, "adam", shapes, dict(weight_decay=0.01), DEV, rounding="half")
+    H.run_steps(opt, orc, params, shapes, 2, torch.float32, 1e-2, DEV, tag="before")
+    homes = [p.data_ptr() for p in params]
+    gen = torch.Generator().manual_seed(99)
+    fresh = [torch.randn(s, generator=gen) * 0.05 for s in shapes]
+    for i in (0, 2):
+        params[i].data = fresh[i].to(DEV)  # new storage
+        orc.params[i].copy_(fresh[i])
+        assert params[i].data_ptr() != homes[i]
+    for k in (3, 4):
+        grads = H.make_grads(shapes, k, torch.float32, 1e-2)
+        for p, g in zip(params, grads):
+            p.grad = g.to(DEV)
+        opt.step()
+        orc.step([g.clone() for g in grads])
+        H.compare(opt, orc, params, f"after rebinding, step {k}")
+    assert [p.data_ptr() for p in params] == homes
+    # a dtype change cannot be absorbed: the slab holds fp32
+    params[1].data = params[1].data.bfloat16()
+    params[1].grad = torch.zeros(shapes[1], device=DEV)
+    with pytest.raises(_lib.HbError, match="dtype"):
+        opt.step()
