@@ -151,7 +151,7 @@ __device__ __forceinline__ float prim_to_f32(uint32_t h) {
 }
 
 // corr / smax, correctly rounded: one Newton correction of c * (1/smax) is exact for every int16 value with
-// smax = 127 and smax = 32767 (checked exhaustively on the host in tests/test_host_arith.py)
+// smax = 127 and smax = 32767 (checked exhaustively on the host in tests/test_host_logic.py)
 template <bool CORR8>
 __device__ __forceinline__ float corr_over_smax(int c) {
   constexpr float smax = CORR8 ? 127.0f : 32767.0f;

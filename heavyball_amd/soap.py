@@ -134,6 +134,8 @@ class SOAP(HBOptimizer):
         if mars or ecc or param_ecc or split or precondition_1d or precond_grad_accum or storage_dtype != "float32" or not merge_dims:
             raise NotImplementedError("SOAP on the HIP kernels: mars, ecc, param_ecc, split, precondition_1d, precond_grad_accum, "
                                       "merge_dims=False and non-fp32 storage are not built")  # fmt: skip
+        if palm not in (use_default, False):
+            raise NotImplementedError("SOAP on the HIP kernels: palm (the beta2 schedule of heavyball/chainable.py:1921-1925) is not built")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
 
     def _run_group(self, gi, group, active):
@@ -200,9 +202,14 @@ class SOAP(HBOptimizer):
                             if m is None:
                                 Q.append(None)
                                 continue
-                            eye = torch.eye(m.shape[-1], dtype=m.dtype, device=m.device)
-                            _, vec = torch.linalg.eigh(m + 1e-30 * eye)  # heavyball/utils.py:1001-1003
-                            Q.append(torch.flip(vec, [-1]).contiguous())
+                            # heavyball/utils.py:1001-1003.  In float64: on a factor with a graded spectrum (singular values of
+                            # the gradient spread over two decades) the vendor's fp32 eigensolver leaves off-diagonal terms of
+                            # 1e-2 of the spectral norm in Q^T GG Q and the eigenvalues out of order, where LAPACK on the CPU,
+                            # which the reference's fixtures come from, leaves 4e-7; in float64 it leaves 1e-15, at
+                            # 0.7 s instead of 0.4 s for an 8192-wide factor, once.
+                            eye = torch.eye(m.shape[-1], dtype=torch.float64, device=m.device)
+                            _, vec = torch.linalg.eigh(m.double() + 1e-30 * eye)
+                            Q.append(torch.flip(vec, [-1]).to(torch.float32).contiguous())
                         st[K_GG], st[K_Q] = GG, Q
                         st.setdefault("is_initialized", set()).update({0, 2, 3})
                         continue

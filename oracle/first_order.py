@@ -317,6 +317,13 @@ def global_rmsnorm_clip(xs: List[Tensor], clip_at=1.0, eps=1e-8) -> List[Tensor]
 # ---------------------------------------------------------------------------------------------------------
 # The step loop of one param group
 # ---------------------------------------------------------------------------------------------------------
+def palm_betas(betas, step: Tensor, beta2_scale: float):
+    """heavyball/chainable.py:1921-1925 (``palm_beta2``, first in the chain: :2693-2694): beta2 = 1 - step ** -beta2_scale
+    on the int64 step tensor, i.e. an fp32 0-d tensor, written back into the group's betas."""
+    beta2 = 1 - step ** -beta2_scale
+    return (betas[0], beta2, *betas[2:])
+
+
 class FirstOrderOracle:
     """AdamW or LaProp over a list of tensors, with the reference's state layout.
 
@@ -350,6 +357,8 @@ class FirstOrderOracle:
         alpha_warmup=None,
         momentum_decay=4e-3,
         decoupled_weight_decay=False,
+        palm=False,
+        beta2_scale=0.8,
     ):
         assert kind in ("adam", "laprop", "adopt", "ademamix", "nadam")
         assert update_clipping is None or kind in ("adam", "laprop"), "update_clipping is restated for AdamW / LaProp only"
@@ -362,6 +371,7 @@ class FirstOrderOracle:
         self.mars_idx = {"adam": 2, "laprop": 2, "ademamix": 2, "adopt": 3, "nadam": 3}[kind]
         self.alpha, self.beta3_warmup, self.alpha_warmup = alpha, beta3_warmup, alpha_warmup
         self.momentum_decay, self.decoupled_weight_decay = momentum_decay, decoupled_weight_decay
+        self.palm, self.beta2_scale = palm, beta2_scale
         if update_clipping is not None:  # heavyball/chainable.py:2676-2684: the fused transform is swapped for the un-fused one
             self.fn_name = {"adam": "scale_by_adam", "laprop": "scale_by_laprop"}[kind]
         # constructor defaults of heavyball/__init__.py:44-80 (AdamW), :740-776 (LaProp), :640-681 (ADOPT), :124-164, :83-121
@@ -419,6 +429,8 @@ class FirstOrderOracle:
         self.state[idx[0]]["step"] = step
         lr = step_lr(self.lr, step, self.warmup_steps)
         rounding = self.rounding.at_step(int(step))
+        if self.palm:
+            self.betas = palm_betas(self.betas, step, self.beta2_scale)
         p = [self.params[i] for i in idx]
         grad = [grads[i] for i in idx]
         update = [g.clone() for g in grad]  # heavyball/chainable.py:2293

@@ -272,6 +272,17 @@ def make_variant_trajectories():
     run_traj("nadam_mars_paramecc", N, dict(mars=True, ecc="bf16+16", param_ecc="bf16+8", momentum_decay=0.1), shapes, torch.float32, 4)
 
 
+def make_palm_trajectories():
+    """``palm=True`` (heavyball/chainable.py:1921-1925, :2693-2694): beta2 = 1 - step ** -beta2_scale, written back into
+    the group's betas each step, ahead of the update transform (and of MARS' index in the state keys)."""
+    shapes = [(4, 8), (16,), (3, 5)]
+    run_traj("adamw_palm", heavyball.AdamW, dict(palm=True, weight_decay=0.01), shapes, torch.float32, 6)
+    run_traj("laprop_palm_ecc", heavyball.LaProp, dict(palm=True, beta2_scale=0.6, ecc="bf16+8"), shapes, torch.bfloat16, 5, grad_scale=1e-3)
+    run_traj("adamw_palm_mars", heavyball.AdamW, dict(palm=True, mars=True), shapes, torch.float32, 4)
+    run_traj("adopt_palm", heavyball.ADOPT, dict(palm=True), shapes, torch.float32, 4)
+    run_traj("nadam_palm", heavyball.NAdam, dict(palm=True), shapes, torch.float32, 4)
+
+
 def make_ns5():
     """Newton-Schulz vectors straight from the reference's functions, the bf16 stochastic round made round-half-up."""
     out = {}
@@ -368,7 +379,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "ns5", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "ns5", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -379,6 +390,8 @@ if __name__ == "__main__":
         make_trajectories()
     if "variants" in which:
         make_variant_trajectories()
+    if "palm" in which:
+        make_palm_trajectories()
     if "ns5" in which:
         make_ns5()
     if "muon" in which:

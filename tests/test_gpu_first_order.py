@@ -87,6 +87,11 @@ CASES = [
     ("nadam_mars_paramecc_coupled_caution", "NAdam", dict(mars=True, ecc="bf16+16", param_ecc="bf16+8", momentum_decay=0.1, weight_decay=0.05,
                                                           caution=True), torch.float32, 1e-2),
     ("nadam_bf16_storage", "NAdam", dict(storage_dtype="bfloat16"), torch.float32, 1e-2),
+    # palm: beta2 = 1 - step ** -beta2_scale (heavyball/chainable.py:1921-1925)
+    ("adamw_palm", "AdamW", dict(palm=True, weight_decay=0.01), torch.float32, 1e-2),
+    ("laprop_palm_ecc_mars", "LaProp", dict(palm=True, beta2_scale=0.6, ecc="bf16+8", mars=True), torch.bfloat16, 1e-3),
+    ("adopt_palm", "ADOPT", dict(palm=True), torch.float32, 1e-2),
+    ("nadam_palm_caution", "NAdam", dict(palm=True, caution=True), torch.float32, 1e-2),
 ]
 
 

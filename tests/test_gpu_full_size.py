@@ -150,6 +150,34 @@ def test_newton_schulz_on_a_llama_layer():
         assert err < 2e-2
 
 
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_legacy_newton_schulz_matches_oracle_on_square_matrices(n):
+    """The legacy schedule (one coefficient triple, the norm taken after the bf16 cast, a second stochastic round;
+    heavyball/utils.py:637-657) applies to square matrices only.  At these sizes the products run on the 256-square
+    tile class with mirrored symmetric tiles, which the small reference vectors (16 and 64 wide) never reach."""
+    from oracle import muon as omuon
+    from oracle.rounding import HalfRounding
+
+    L = _lib.lib()
+    print("case legacy", n, flush=True)
+    torch.manual_seed(40 + n)
+    g = torch.randn(n, n, device=DEV) * 1e-2
+    nb = ctypes.c_int64()
+    _lib.check(L.hb_ns5_workspace_bytes(n, n, ctypes.byref(nb)))
+    ws = torch.empty(nb.value, dtype=torch.uint8, device=DEV)
+    out = torch.empty_like(g)
+    arr = (ctypes.c_float * 15)(*muon.ns_coefficients(muon.LEGACY_COEFFS))
+    _lib.check(L.hb_ns5(g.data_ptr(), out.data_ptr(), n, n, arr, _lib.NS_LEGACY, 1e-7, 1.0, _lib.RNG_HALF, 1, 1, 0, ws.data_ptr(), nb.value, None))
+    torch.cuda.synchronize()
+    want = omuon.orthogonal(g.cpu().clone(), HalfRounding(), 0, mode="legacy_newtonschulz")
+    err = ((out.cpu().double() - want.double()).norm() / want.double().norm()).item()
+    print("legacy", n, "vs oracle, rel fro", err, flush=True)
+    assert err < 2e-2
+    # the legacy triple maps singular values into a band around 1 as well (wider than the default schedule's)
+    sv = torch.linalg.eigvalsh((out @ out.T).double()).clamp(min=0).sqrt()
+    assert sv.max() < 1.35 and (sv > 0.6).double().mean() > 0.85
+
+
 def test_soap_products_and_orthonormalisation_at_full_size():
     """[2048, 8192]: an orthonormal basis from hb_orthonormalize_f32 on each side, rotate and rotate back (four GEMMs in
     all four operand orientations) returns the matrix; the factor product is symmetric and matches a float64 row."""

@@ -147,3 +147,29 @@ def test_ns_coefficients_follow_cpu_scalar_rounding():
     assert len(c) == 15
     assert c[0] == 4.09375 and c[1] == -6.90625  # a, b rounded to bf16 (in-place bf16 add casts its scalar)
     assert abs(c[2] - 2.9270) < 1e-6 and c[2] != float(torch.tensor(2.9270).bfloat16())  # c stays fp32
+
+
+def test_corr_over_smax_newton_step_is_correctly_rounded_for_every_correction():
+    """The kernels decode ``corr / smax`` (heavyball/utils.py:1298, an fp32 divide) as q0 = c * r, q = fma(fma(-q0, smax, c), r, q0)
+    with r = fl32(1 / smax): exhaustively, for every int16 value and both smax (127, 32767), that equals the correctly
+    rounded quotient.  numpy has no fma; the two fused steps are evaluated in float64, where products of fp32 values
+    are exact and each sum carries one rounding to fp32 that cannot be a double rounding (the exact results have at most
+    48 + 24 significant bits only in the first step, whose result c - q0 * smax is exactly representable)."""
+    import numpy as np
+
+    c = np.arange(-32768, 32768, dtype=np.int64)
+    for smax in (127.0, 32767.0):
+        cf = c.astype(np.float32)
+        sm = np.float32(smax)
+        r = np.float32(1.0) / sm
+        want = cf / sm  # IEEE fp32 division
+        q0 = cf * r
+        rem = (cf.astype(np.float64) - q0.astype(np.float64) * np.float64(sm)).astype(np.float32)  # exact: |rem| < ulp(c), few bits
+        assert np.array_equal(rem.astype(np.float64), cf.astype(np.float64) - q0.astype(np.float64) * np.float64(sm))
+        exact = q0.astype(np.float64) + rem.astype(np.float64) * np.float64(r)  # 24 x 24-bit product plus a 24-bit value
+        q = exact.astype(np.float32)
+        # the float64 sum is itself rounded (to 53 bits) before the rounding to fp32: where it falls within one float64 ulp
+        # of an fp32 rounding boundary the two-step result could differ from the fused one; no case comes that close
+        mid = (q.astype(np.float64) + np.nextafter(q, np.where(exact > q, np.float32(np.inf), np.float32(-np.inf))).astype(np.float64)) / 2
+        assert (np.abs(exact - mid) > 4 * np.spacing(np.abs(exact))).all()
+        assert np.array_equal(q.view(np.uint32), want.view(np.uint32)), smax
