@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer-step hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c3|c3s|c3nc|c2l|adopt|ademamix|nadam] [--no-cpu] [--soap-products]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c3|c3s|c3nc|c2l|adopt|ademamix|nadam] [--no-cpu] [--no-muon]
+                    [--no-soap] [--no-8b] [--soap-products]
 
 Default workload (the headline configuration, "c2"): LaProp with ecc="bf16+8" on a GPT-2-small-shaped parameter set
 (147 tensors, 123,653,376 elements), fp32 parameters, bf16 gradients ~ N(0, 1e-3), synthetic data generated on the
@@ -10,7 +11,10 @@ device.  A "step" is one ``optimizer.step()`` over the whole set with the gradie
 Prints ONE JSON line.  ``value`` is the wall-clock ms per step of ``optimizer.step()`` (host overhead included);
 ``roofline`` is computed from the fused kernel's own duration, measured with HIP events on the launch stream around
 back-to-back launches of ``hb_fused_step``; ``cpu_baseline`` is the CPU oracle (an op-for-op restatement of the
-reference's eager path) timed on this machine's host cores on a bounded sample and scaled to the full element count.
+reference's eager path) timed on this machine's host cores: the whole of configuration c2, three steps after a warm-up.
+Beside the headline the line carries the reference's own micro-benchmark protocol (``adamw_reference_script``), Muon's
+Newton-Schulz (``ns5``), SOAP (``soap``) and, when 200 GiB of device memory are free, the Llama-3-8B-shaped parameter set
+under LaProp and under AdamW with MARS, caution, ECC states and ECC parameters (``llama8b``), each with its own roofline.
 """
 
 import argparse
@@ -77,15 +81,12 @@ def cpu_baseline(cfg_name, total_elems):
     from oracle.rounding import TorchRounding
 
     cls, kwargs, shapes, gdt, gstd, _, _ = CONFIGS[cfg_name]
-    if cfg_name == "c2":
-        sample = shapes[:12] + [(4096, 768)]
-        what = "one transformer layer (12 tensors) + a [4096,768] slice of the embedding"
-    elif cfg_name in ("c3", "c3s", "c3nc", "c2l"):
+    if cfg_name in ("c3", "c3s", "c3nc", "c2l"):
         sample = [(1024, 4096), (1024, 4096), (4096,), (4096,), (2048, 4096)]
         what = "k/v projections, two norms and a [2048,4096] slice of one Llama-3-8B layer"
     else:
         sample = shapes
-        what = "the full config"
+        what = "the full config (every tensor, every element)"
     n = sum(int(torch.Size(s).numel()) for s in sample)
     gen = torch.Generator().manual_seed(0)
     params = [torch.randn(s, generator=gen) * 0.02 for s in sample]
@@ -98,6 +99,8 @@ def cpu_baseline(cfg_name, total_elems):
         t0 = time.perf_counter()
         orc.step(grads)
         times.append(time.perf_counter() - t0)
+        if sum(times) > 25.0 and len(times) >= 2:  # bounded: about half a minute of CPU work at most
+            break
     per_step = statistics.median(times[1:])
     scaled_ms = per_step * 1e3 * total_elems / n
     return {
@@ -105,13 +108,97 @@ def cpu_baseline(cfg_name, total_elems):
         "unit": "ms/step",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{what}: {n} elements, median of 3 steps after 1 warm-up = {per_step * 1e3:.1f} ms, "
+        "sample": f"{what}: {n} elements, median of {len(times) - 1} steps after 1 warm-up = {per_step * 1e3:.1f} ms, "
                   f"scaled linearly to {total_elems} elements; torch {torch.__version__} eager CPU ops in the reference's order",
         "elements_per_s": round(n / per_step, 1),
         # the lines of torch.__config__.parallel_info() that name the threading back end and its thread counts
         "parallel_info": "; ".join(ln.strip() for ln in torch.__config__.parallel_info().splitlines()
                                    if any(k in ln for k in ("ATen parallel backend", "get_num_threads", "max_threads", "num_interop"))),
     }  # fmt: skip
+
+
+# hb::fused_step_kernel's HBM traffic per launch on config c2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
+# against a copy of known size (not measured in this run): the value and the file that documents it
+C2_TRAFFIC_FROM_PROFILE = (2722.5e6, "profiles/fused_step_c2_hbm_traffic.txt")
+
+
+def bench_first_order(cfg_name, steps, warmup, kernel_launches, rounding="philox"):
+    """One first-order configuration: ``steps`` calls of ``optimizer.step()`` over the whole parameter set with the
+    gradients resident in HBM (wall clock, host overhead included), then the kernel alone: HIP events on the launch stream
+    around back-to-back ``hb_fused_step`` calls on the same descriptor.  Returns the fields of the JSON line."""
+    import torch
+
+    import heavyball_amd
+    from heavyball_amd import _lib
+
+    dev = torch.device("cuda:0")
+    cls_name, kwargs, shapes, gdt, gstd, bytes_per_elem, label = CONFIGS[cfg_name]
+    gdtype = getattr(torch, gdt)
+    total = sum(int(torch.Size(s).numel()) for s in shapes)
+
+    torch.manual_seed(0)
+    params = []
+    for s in shapes:
+        p = torch.nn.Parameter(torch.randn(s, device=dev) * 0.02)
+        p.grad_dtype = None
+        params.append(p)
+    opt = getattr(heavyball_amd, cls_name)(params, **kwargs)
+    opt.rounding = rounding
+    # gradient sets resident in HBM before the timed region; cycled if memory is tight
+    n_sets = 4 if total < 1_000_000_000 else 1
+    grad_sets = [[(torch.randn(s, device=dev) * gstd).to(gdtype) for s in shapes] for _ in range(n_sets)]
+
+    def one_step(k):
+        gs = grad_sets[k % n_sets]
+        for p, g in zip(params, gs):
+            p.grad = g
+        opt.step()
+
+    for k in range(warmup):
+        one_step(k)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        one_step(k)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+
+    # kernel-only duration: HIP events on the launch stream around back-to-back launches of the same descriptor
+    desc, _ = opt._last_launch
+    L = _lib.lib()
+    stream = torch.cuda.current_stream(dev)
+    for _ in range(3):
+        _lib.check(L.hb_fused_step(desc, stream.cuda_stream))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(kernel_launches):
+        _lib.check(L.hb_fused_step(desc, stream.cuda_stream))
+    e1.record(stream)
+    torch.cuda.synchronize()
+    kernel_ms = e0.elapsed_time(e1) / kernel_launches
+    algo_bytes = bytes_per_elem * total
+    achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": C2_TRAFFIC_FROM_PROFILE[0] if cfg_name == "c2" else None,
+        "algorithmic_bytes_per_launch": algo_bytes,
+        "kernel": "hb::fused_step_kernel (all launches of one hb_fused_step call)",
+    }
+    if cfg_name == "c2":
+        roofline["traffic_source"] = f"{C2_TRAFFIC_FROM_PROFILE[1]} (hardware counters of an earlier run of this command, not of this run)"
+    del grad_sets, params
+    return {
+        "config": {"workload": label, "elements": total, "tensors": len(shapes), "rounding": opt.rounding, "name": cfg_name},
+        "ms_per_step": round(ms_per_step, 4),
+        "kernel_ms": round(kernel_ms, 4),
+        "elements_per_s": round(total / (ms_per_step * 1e-3), 1),
+        "roofline": roofline,
+    }
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0
@@ -422,6 +509,7 @@ def main():
     ap.add_argument("--rounding", default="philox", choices=["philox", "half"])
     ap.add_argument("--no-muon", action="store_true", help="skip the Muon / Newton-Schulz leg (Benchmark configuration 4)")
     ap.add_argument("--no-soap", action="store_true", help="skip the SOAP leg (Benchmark configuration 5)")
+    ap.add_argument("--no-8b", action="store_true", help="skip the legs on the Llama-3-8B-shaped parameter set (112 GB of device memory)")
     ap.add_argument("--soap-products", action="store_true",
                     help="run only the 18 fp32 products of one SOAP step on random operands (for hardware-counter runs) and exit")
     ap.add_argument("--calibrate", action="store_true",
@@ -443,84 +531,29 @@ def main():
     if args.soap_products:
         bench_soap_products()
         return
-    dev = torch.device("cuda:0")
-    cls_name, kwargs, shapes, gdt, gstd, bytes_per_elem, label = CONFIGS[args.config]
-    gdtype = getattr(torch, gdt)
-    total = sum(int(torch.Size(s).numel()) for s in shapes)
-
-    torch.manual_seed(0)
-    params = []
-    for s in shapes:
-        p = torch.nn.Parameter(torch.randn(s, device=dev) * 0.02)
-        p.grad_dtype = None
-        params.append(p)
-    opt = getattr(heavyball_amd, cls_name)(params, **kwargs)
-    opt.rounding = args.rounding
-    # gradient sets resident in HBM before the timed region; cycled if memory is tight
-    n_sets = 4 if total < 1_000_000_000 else 1
-    grad_sets = [[(torch.randn(s, device=dev) * gstd).to(gdtype) for s in shapes] for _ in range(n_sets)]
-
-    def one_step(k):
-        gs = grad_sets[k % n_sets]
-        for p, g in zip(params, gs):
-            p.grad = g
-        opt.step()
-
-    for k in range(args.warmup):
-        one_step(k)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        one_step(k)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-
-    # kernel-only duration: HIP events on the launch stream around back-to-back launches of the same descriptor
-    desc, _ = opt._last_launch
-    L = _lib.lib()
-    stream = torch.cuda.current_stream(dev)
-    n_launch = args.kernel_launches
-    for _ in range(3):
-        _lib.check(L.hb_fused_step(desc, stream.cuda_stream))
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(n_launch):
-        _lib.check(L.hb_fused_step(desc, stream.cuda_stream))
-    e1.record(stream)
-    torch.cuda.synchronize()
-    kernel_ms = e0.elapsed_time(e1) / n_launch
-    algo_bytes = bytes_per_elem * total
-    achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
-
+    first = bench_first_order(args.config, args.steps, args.warmup, args.kernel_launches, args.rounding)
+    total = first["config"]["elements"]
     out = {
         "metric": METRIC,
-        "value": round(ms_per_step, 4),
+        "value": first["ms_per_step"],
         "unit": "ms/step",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": first["ms_per_step"],
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": label, "elements": total, "tensors": len(shapes), "rounding": opt.rounding, "name": args.config},
-        "elements_per_s": round(total / (ms_per_step * 1e-3), 1),
-        "kernel_ms": round(kernel_ms, 4),
-        "roofline": {
-            "bound": "hbm",
-            "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled against hb_copy_probe (profiles/): config c2 only
-            "traffic": 2723.8e6 if args.config == "c2" else None,
-            "algorithmic_bytes_per_launch": algo_bytes,
-            "kernel": "hb::fused_step_kernel (all launches of one hb_fused_step call)",
-        },
+        "config": first["config"],
+        "elements_per_s": first["elements_per_s"],
+        "kernel_ms": first["kernel_ms"],
+        "roofline": first["roofline"],
     }
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+    stream = torch.cuda.current_stream(dev)
     if args.calibrate:
         a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         b = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -529,7 +562,6 @@ def main():
             _lib.check(L.hb_copy_probe(a.data_ptr(), b.data_ptr(), 1 << 30, stream.cuda_stream))
         torch.cuda.synchronize()
         del a, b
-    del grad_sets, params, opt
     torch.cuda.empty_cache()
     out["adamw_reference_script"] = bench_reference_script()
     torch.cuda.empty_cache()
@@ -540,6 +572,18 @@ def main():
         out["soap"] = bench_soap()
         torch.cuda.empty_cache()
         out["soap"]["default_max_precond_dim"] = bench_soap_default_dim()
+    if args.config == "c2" and not args.no_8b:
+        # the 8B-shaped parameter set (benchmark configuration 3), under the headline's optimizer and under its own
+        torch.cuda.empty_cache()
+        free, _ = torch.cuda.mem_get_info(dev)
+        if free < 200 * 2**30:
+            out["llama8b"] = {"skipped": f"{free / 2**30:.0f} GiB of device memory free, the 8B-shaped set wants 200"}
+        else:
+            out["llama8b"] = {}
+            for name in ("c2l", "c3"):
+                leg = bench_first_order(name, 5, 2, 5, args.rounding)
+                out["llama8b"][name] = {k: leg[k] for k in ("config", "ms_per_step", "kernel_ms", "elements_per_s", "roofline")}
+                torch.cuda.empty_cache()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.config, total)
     print(json.dumps(out))
