@@ -61,13 +61,15 @@ __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs 
       const int64_t idx = flat0 + e;
       Raw ru, rp;
       float u[8], p[8], g[8];
-      raw_load<HB_FMT_F32>(ru, HB_FMT_F32, a.m, nullptr, idx);
+      if (a.sf == HB_FMT_BF16) raw_load<HB_FMT_BF16>(ru, HB_FMT_BF16, a.m, nullptr, idx);  // the update as a bf16 slab
+      else raw_load<HB_FMT_F32>(ru, HB_FMT_F32, a.m, nullptr, idx);
       if (!kCount) raw_load<PF>(rp, pf, a.param, a.param_corr, idx);
       if (CAUTION != kNoCaution) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) g[j] = e + j < valid ? load_elem(gbase, a.gf, g0 + e + j) : 0.0f;
       }
-      raw_decode<HB_FMT_F32>(ru, HB_FMT_F32, u);
+      if (a.sf == HB_FMT_BF16) raw_decode<HB_FMT_BF16>(ru, HB_FMT_BF16, u);
+      else raw_decode<HB_FMT_F32>(ru, HB_FMT_F32, u);
       if (!kCount) raw_decode<PF>(rp, pf, p);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -127,8 +129,11 @@ static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states, bool ne
   if (fmt_is_ecc(d->param_fmt) && (!d->param_corr || !aligned16(d->param_corr)))
     return set_error(HB_EINVAL, "param_corr required (16-byte aligned) for an ECC param_fmt");
   const bool caution = (d->flags & HB_FLAG_CAUTION) != 0;
-  if ((d->flags & HB_FLAG_UPDATE_ONLY) && (caution || d->param_fmt != HB_FMT_F32))
-    return set_error(HB_EINVAL, "HB_FLAG_UPDATE_ONLY writes an fp32 update slab and takes no caution flag");
+  if ((d->flags & HB_FLAG_UPDATE_ONLY) && (caution || (d->update_out == nullptr && d->param_fmt != HB_FMT_F32) ||
+                                           (d->update_out != nullptr && !aligned16(d->update_out))))
+    return set_error(HB_EINVAL, "HB_FLAG_UPDATE_ONLY writes an fp32 update slab (update_out, or param with param_fmt F32) and takes no caution flag");
+  if ((d->flags & HB_FLAG_MARS_ONLY) && (!(d->flags & HB_FLAG_MARS) || caution || d->param_fmt != HB_FMT_F32 || !need_states))
+    return set_error(HB_EINVAL, "HB_FLAG_MARS_ONLY goes with HB_FLAG_MARS, writes an fp32 slab and takes no caution flag");
   const bool need_grad = need_states || caution;
   if (need_grad) {
     if (!fmt_ok_grad(d->grad_fmt)) return set_error(HB_EINVAL, "bad grad_fmt");
@@ -141,16 +146,17 @@ static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states, bool ne
     if ((d->flags & HB_FLAG_ADOPT_WARMUP) && (d->algo != HB_ALGO_ADOPT || caution || (d->flags & HB_FLAG_UPDATE_ONLY)))
       return set_error(HB_EINVAL, "HB_FLAG_ADOPT_WARMUP goes with HB_ALGO_ADOPT alone and takes no caution");
     if ((d->flags & HB_FLAG_COUPLED_WD) && d->algo != HB_ALGO_NADAM) return set_error(HB_EINVAL, "HB_FLAG_COUPLED_WD goes with HB_ALGO_NADAM");
-    if ((d->flags & HB_FLAG_UPDATE_ONLY) && d->algo > HB_ALGO_LAPROP)
-      return set_error(HB_EINVAL, "HB_FLAG_UPDATE_ONLY is built for HB_ALGO_ADAM and HB_ALGO_LAPROP");
+    if ((d->flags & HB_FLAG_UPDATE_ONLY) && (d->flags & HB_FLAG_COUPLED_WD) && d->update_out == nullptr)
+      return set_error(HB_EINVAL, "HB_FLAG_UPDATE_ONLY with HB_FLAG_COUPLED_WD reads the parameters: give the update its own slab in update_out");
     if (d->algo == HB_ALGO_NADAM && !d->tensor_scalars) return set_error(HB_EINVAL, "tensor_scalars required with HB_ALGO_NADAM");
     if (!fmt_ok_state(d->state_fmt) || d->state_fmt > HB_FMT_ECC_F16_16) return set_error(HB_EINVAL, "bad state_fmt");
     const bool ecc = fmt_is_ecc(d->state_fmt);
-    if (!d->exp_avg || !d->exp_avg_sq || !aligned16(d->exp_avg) || !aligned16(d->exp_avg_sq))
+    const bool mars_only = (d->flags & HB_FLAG_MARS_ONLY) != 0;
+    if (!mars_only && (!d->exp_avg || !d->exp_avg_sq || !aligned16(d->exp_avg) || !aligned16(d->exp_avg_sq)))
       return set_error(HB_EINVAL, "exp_avg / exp_avg_sq must be 16-byte aligned device pointers");
-    if (ecc && (!d->exp_avg_corr || !d->exp_avg_sq_corr || !aligned16(d->exp_avg_corr) || !aligned16(d->exp_avg_sq_corr)))
+    if (!mars_only && ecc && (!d->exp_avg_corr || !d->exp_avg_sq_corr || !aligned16(d->exp_avg_corr) || !aligned16(d->exp_avg_sq_corr)))
       return set_error(HB_EINVAL, "state corrections required (16-byte aligned) for an ECC state_fmt");
-    if (d->algo == HB_ALGO_ADEMAMIX) {
+    if (d->algo == HB_ALGO_ADEMAMIX && !mars_only) {
       if (!d->exp_avg_slow || !aligned16(d->exp_avg_slow)) return set_error(HB_EINVAL, "exp_avg_slow required with HB_ALGO_ADEMAMIX");
       if (ecc && (!d->exp_avg_slow_corr || !aligned16(d->exp_avg_slow_corr))) return set_error(HB_EINVAL, "exp_avg_slow_corr required");
     }
@@ -158,8 +164,8 @@ static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states, bool ne
       if (!d->old_grad || !aligned16(d->old_grad)) return set_error(HB_EINVAL, "old_grad required with HB_FLAG_MARS");
       if (ecc && (!d->old_grad_corr || !aligned16(d->old_grad_corr))) return set_error(HB_EINVAL, "old_grad_corr required");
     }
-  } else if (!d->exp_avg || !aligned16(d->exp_avg)) {
-    return set_error(HB_EINVAL, "hb_update_param reads the fp32 update from exp_avg");
+  } else if (!d->exp_avg || !aligned16(d->exp_avg) || (d->state_fmt != HB_FMT_F32 && d->state_fmt != HB_FMT_BF16)) {
+    return set_error(HB_EINVAL, "hb_update_param reads the update from exp_avg, an fp32 or (state_fmt HB_FMT_BF16) bf16 slab");
   }
   if (d->rng_mode != HB_RNG_HALF && d->rng_mode != HB_RNG_PHILOX) return set_error(HB_EINVAL, "bad rng_mode");
   a.param = static_cast<char*>(d->param);
@@ -175,6 +181,7 @@ static int fill_args(const HbStepDesc* d, StepArgs& a, bool need_states, bool ne
   a.s3 = static_cast<char*>(d->exp_avg_slow);
   a.s3_corr = static_cast<char*>(d->exp_avg_slow_corr);
   a.tscal = d->tensor_scalars;
+  a.upd = static_cast<char*>(d->update_out);
   a.offsets = d->offsets;
   a.numel = d->numel;
   a.chunks = reinterpret_cast<const int2*>(d->chunks);

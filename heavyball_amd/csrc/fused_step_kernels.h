@@ -47,6 +47,7 @@ struct StepArgs {
   char* og_corr;
   char* s3;  // AdEMAMix: slow momentum
   char* s3_corr;
+  char* upd;           // HB_FLAG_UPDATE_ONLY: fp32 slab that takes the update (null: a.param does)
   const float* tscal;  // NAdam: two weights per tensor
   const int64_t* offsets;
   const int64_t* numel;
@@ -85,6 +86,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   const bool cautious_wd = (a.flags & HB_FLAG_CAUTIOUS_WD) != 0;
   const bool update_only = (a.flags & HB_FLAG_UPDATE_ONLY) != 0;
   const bool write_grad = MARS && !kCount && (a.flags & HB_FLAG_WRITE_GRAD) != 0;
+  const bool mars_only = MARS && (a.flags & HB_FLAG_MARS_ONLY) != 0;  // the prologue alone: corrected gradient -> a.param (fp32)
   const bool state_rounds = sf != HB_FMT_F32;
   // raw gradient -> old_grad: exact (no noise needed) when both are bf16, or the target is fp32
   const bool og_rounds = MARS && state_rounds && !(gf == HB_FMT_BF16 && fmt_prim_bf16(sf));
@@ -109,11 +111,15 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
         for (int j = 0; j < kE; ++j) gtail[k][j] = e + j < valid ? load_elem(gbase, gf, g0 + e + j) : 0.0f;
       }
       if (kAdopt) rm[k] = rp[k] = RawT<kE>{};
-      if (!kAdopt || !warmup) raw_load<SF>(rm[k], sf, a.m, a.m_corr, idx);
-      if (kNeedV) raw_load<SF>(rv[k], sf, a.v, a.v_corr, idx);
-      if (kMix) raw_load<SF>(rs[k], sf, a.s3, a.s3_corr, idx);
       if (MARS) raw_load<SF>(ro[k], sf, a.og, a.og_corr, idx);
-      if ((!kCount && (!kAdopt || !warmup)) || (kNadam && coupled)) raw_load<PF>(rp[k], pf, a.param, a.param_corr, idx);
+      if (mars_only) {
+        rm[k] = rv[k] = rs[k] = rp[k] = RawT<kE>{};
+      } else {
+        if (!kAdopt || !warmup) raw_load<SF>(rm[k], sf, a.m, a.m_corr, idx);
+        if (kNeedV) raw_load<SF>(rv[k], sf, a.v, a.v_corr, idx);
+        if (kMix) raw_load<SF>(rs[k], sf, a.s3, a.s3_corr, idx);
+        if ((!kCount && (!kAdopt || !warmup)) || (kNadam && coupled)) raw_load<PF>(rp[k], pf, a.param, a.param_corr, idx);
+      }
     }
   };
   for_each_index(fetch, std::make_integer_sequence<int, kGroups>{});
@@ -161,6 +167,11 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
 #pragma unroll
           for (int j = 0; j < kE; ++j)
             if (FULL || e + j < valid) store_elem(const_cast<char*>(gbase), gf, g0 + e + j, g[j]);
+        }
+        if (mars_only) {
+          raw_encode<HB_FMT_F32>(w, HB_FMT_F32, g, Noise<kE>{});
+          raw_store<HB_FMT_F32>(w, HB_FMT_F32, a.param, nullptr, idx);
+          return;
         }
       }
     }
@@ -214,7 +225,15 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
     }
 
     if (!kCount) {
-      if (update_only) {  // un-fused transform: the update itself is the output
+      if (update_only) {  // un-fused transform: the update itself is the output, in the precision of the reference's update buffer
+        if (gf == HB_FMT_BF16) {
+          const Noise<kE> rn_u = a.rng.noise<kE>(idx, HB_STREAM_UPDATE);
+#pragma unroll
+          for (int j = 0; j < kE; ++j) u[j] = bf16_to_f32(sr_bf16(u[j], rn_u.bits16(j)));
+        } else if (gf == HB_FMT_F16) {
+#pragma unroll
+          for (int j = 0; j < kE; ++j) u[j] = f16_to_f32(f32_to_f16_rne(u[j]));
+        }
 #pragma unroll
         for (int j = 0; j < kE; ++j) p[j] = u[j];
       } else if (cautious_wd) {  // heavyball/utils.py:2388-2389
@@ -241,7 +260,10 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
         raw_encode<SF>(w, sf, sl, rn);
         raw_store<SF>(w, sf, a.s3, a.s3_corr, idx);
       }
-      if (!kAdopt || !warmup) {
+      if (update_only && a.upd != nullptr) {
+        raw_encode<HB_FMT_F32>(w, HB_FMT_F32, p, Noise<kE>{});
+        raw_store<HB_FMT_F32>(w, HB_FMT_F32, a.upd, nullptr, idx);
+      } else if (!kAdopt || !warmup) {
         if (!MARS && pf != HB_FMT_F32) rn_p = a.rng.noise<kE>(idx, HB_STREAM_PARAM);
         raw_encode<PF>(w, pf, p, rn_p);
         raw_store<PF>(w, pf, a.param, a.param_corr, idx);

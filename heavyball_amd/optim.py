@@ -465,7 +465,30 @@ class HBOptimizer(torch.optim.Optimizer):
                                       n_chunks, current_stream_ptr(b.device)), "hb_scale")  # fmt: skip
         return plan, scales
 
-    def _clip_gradients(self, L, group, buckets, step):
+    def _mars_prologue(self, L, group, b, lst, gdt, step, mars_a, mars_oma, state_fmt, k_o):
+        """MARS alone over one bucket: ``mars_old_grad`` takes the raw gradients, the corrected ones (rounded to the gradient
+        dtype) land in the fp32 slab role ``_clip``."""
+        offsets, numel = b.slab.meta()
+        chunks, n_chunks = b.slab.chunks(tuple(i for i, _ in lst))
+        ptrs = [0] * len(b.params)
+        for i, g in lst:
+            ptrs[i] = g.data_ptr()
+        table = b.grad_ptr_table(gdt, ptrs)
+        out = b.slab.role("_clip", torch.float32)
+        d = _lib.HbStepDesc()
+        d.param, d.param_fmt = out.data_ptr(), _lib.FMT_F32
+        d.grad, d.grad_ptrs, d.grad_fmt = None, table.data_ptr(), _PLAIN_FMT[gdt]
+        d.old_grad, d.old_grad_corr, d.state_fmt = b.slab.ptr(k_o), b.slab.ptr(k_o + "::ecc"), state_fmt
+        d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
+        d.n_chunks, d.n_tensors = n_chunks, len(b.params)
+        d.algo, d.flags = _lib.ALGO_ADAM, _lib.FLAG_MARS | _lib.FLAG_MARS_ONLY  # the prologue is the same for every algorithm
+        d.mars_a, d.one_minus_mars_a = mars_a, mars_oma
+        d.rng_mode, d.step, d.seed = self._rng_mode(), int(step) & 0xFFFFFFFF, self.rng_seed
+        with torch.cuda.device(b.device):
+            _lib.check(L.hb_fused_step(d, current_stream_ptr(b.device)), "hb_fused_step (MARS prologue)")
+        self._last_launch = (d, (table, chunks, offsets, numel))
+
+    def _clip_gradients(self, L, group, buckets, step, gathered=False):
         """``gradient_clipping`` (heavyball/chainable.py:2696-2699): the gradients of the group are gathered into the fp32
         slab role ``_clip``, clipped there (``_clip_role``) and, for bf16 gradients, rounded back to bf16 the way
         ``copy_stochastic_`` does (``hb_sr_bf16``).  ``buckets``: [(bucket, [(index, gradient)], gradient dtype)].  Returns,
@@ -475,8 +498,9 @@ class HBOptimizer(torch.optim.Optimizer):
             if gdt not in (torch.float32, torch.bfloat16):
                 raise NotImplementedError(f"gradient_clipping with {gdt} gradients")
             b.slab.role("_clip", torch.float32)
-            for i, g in lst:
-                b.slab.view("_clip", i).copy_(g)
+            if not gathered:  # otherwise an earlier pass (MARS) has left the gradients in the role
+                for i, g in lst:
+                    b.slab.view("_clip", i).copy_(g)
         keep = self._clip_role(L, self.gradient_clipping, "_clip", [(b, [i for i, _ in lst]) for b, lst, _ in buckets])
         result = []
         for b, lst, gdt in buckets:
@@ -666,16 +690,14 @@ class FirstOrder(HBOptimizer):
 
     def _run_group(self, gi, group, active):
         unfused = self.update_clipping is not None
-        if unfused and self._algo not in (_lib.ALGO_ADAM, _lib.ALGO_LAPROP):
-            raise NotImplementedError(f"update_clipping on {type(self).__name__} (its un-fused transform is not built)")
-        if unfused and any(g.dtype != torch.float32 for _, g in active) and not self.promote:
-            raise NotImplementedError("update_clipping with 16-bit gradients (the reference rounds the update to their dtype first)")
-        if self.gradient_clipping is not None and group.get("mars", False):
-            raise NotImplementedError("gradient_clipping together with mars (the clip sits between MARS and the fused transform)")
+        if unfused and any(g.dtype == torch.float16 for _, g in active) and not self.promote:
+            raise NotImplementedError("update_clipping with float16 gradients (the clipped update is re-rounded to bfloat16 or kept in float32)")
         L = _lib.lib()
         step = group["step"]
         lr = f32(group["lr"])
         scal = self._step_scalars(group, step)
+        if unfused and self._algo == _lib.ALGO_ADOPT:
+            scal["eps"] = float(f32(1e-8))  # heavyball/chainable.py:1014-1023 passes no eps to utils.adopt: its default
         decay_py, decay_flags = self._decay(group)
         decay = f32(decay_py)
         omdl = float(1 - decay * lr)
@@ -729,15 +751,28 @@ class FirstOrder(HBOptimizer):
                 if lst is None:
                     lst = by_dtype[dt] = []
                 lst.append((i, g))
-            if self.gradient_clipping is not None and len(by_dtype) > 1:
-                raise NotImplementedError("gradient_clipping with gradients of several dtypes in one bucket")
+            if (self.gradient_clipping is not None or unfused) and len(by_dtype) > 1:
+                raise NotImplementedError("gradient_clipping / update_clipping with gradients of several dtypes in one bucket")
             for gdt, lst in by_dtype.items():
                 lst.sort(key=lambda t: t[0])
                 work.append((b, lst, gdt))
-        clipped = self._clip_gradients(L, group, work, step) if self.gradient_clipping is not None else [None] * len(work)
+        if self.gradient_clipping is not None and mars:
+            # heavyball/chainable.py:2694-2699: MARS, then the clip, then the transform.  The prologue runs as a pass of its
+            # own (HB_FLAG_MARS_ONLY) that leaves the corrected gradients in the fp32 role "_clip"; the step proper then
+            # runs without the MARS flag on the clipped slab
+            for b, lst, gdt in work:
+                self._mars_prologue(L, group, b, lst, gdt, step, mars_a, mars_oma, state_fmt, k_o)
+            flags &= ~(_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD)
+            mars = False
+            clipped = self._clip_gradients(L, group, work, step, gathered=True)
+        elif self.gradient_clipping is not None:
+            clipped = self._clip_gradients(L, group, work, step)
+        else:
+            clipped = [None] * len(work)
         if not self._begin_step(group, work):  # ADOPT's warm-up: only exp_avg_sq moves (and MARS' old gradient)
             flags = (flags & (_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD)) | _lib.FLAG_ADOPT_WARMUP
             scal = dict(scal, a2=1.0, one_minus_a2=0.0)
+            unfused = False  # the warm-up skips the rest of the chain (WarmupGuard, heavyball/chainable.py:597-610)
 
         for (b, lst, gdt), clip in zip(work, clipped):
             offsets, numel = b.slab.meta()
@@ -776,8 +811,12 @@ class FirstOrder(HBOptimizer):
                 # heavyball/chainable.py:2676-2684: with update_clipping the chain is scale_by_* -> clip -> update_param_.
                 # The step kernel only advances the moments and writes the update into the fp32 role "_update".
                 b.slab.role("_update", torch.float32)
-                d.param, d.param_corr, d.param_fmt = b.slab.ptr("_update"), None, _lib.FMT_F32
-                d.flags = (flags & (_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD)) | _lib.FLAG_UPDATE_ONLY
+                d.update_out = b.slab.ptr("_update")
+                d.flags = (flags & (_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD | _lib.FLAG_COUPLED_WD)) | _lib.FLAG_UPDATE_ONLY
+                if mars and group["caution"]:
+                    # the chain's tail compares the clipped update with the gradient as MARS left it (chainable.py:646 writes the
+                    # corrected gradient into the gradient buffer): the step kernel has to write it there
+                    d.flags |= _lib.FLAG_WRITE_GRAD
                 d.caution_count = None
             with torch.cuda.device(b.device):
                 rc = L.hb_fused_step(d, current_stream_ptr(b.device))
@@ -788,16 +827,24 @@ class FirstOrder(HBOptimizer):
         keep = self._clip_updates(L, [(b, [i for i, _ in lst]) for b, lst, _ in work])
         decay_py = group["weight_decay"]  # update_param_ keeps decay a python float (heavyball/utils.py:2393-2406)
         for b, lst, gdt in work:
+            upd_role, upd_fmt = "_update", _lib.FMT_F32
+            if gdt == torch.bfloat16:
+                # the clip writes its result back into the bf16 update buffer through copy_stochastic_ (heavyball/utils.py:3231)
+                wide, narrow = b.slab.role("_update", torch.float32), b.slab.role("_update16", torch.bfloat16)
+                with torch.cuda.device(b.device):
+                    _lib.check(L.hb_sr_bf16(wide.data_ptr(), narrow.data_ptr(), wide.numel(), self._rng_mode(), self.rng_seed,
+                                            int(step) & 0xFFFFFFFF, _lib.STREAM_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
+                upd_role, upd_fmt = "_update16", _lib.FMT_BF16
             offsets, numel = b.slab.meta()
             chunks, n_chunks = b.slab.chunks(tuple(i for i, _ in lst))
             ptrs = [0] * len(b.params)
             for i, g in lst:
                 ptrs[i] = g.data_ptr()
-            table = b.grad_ptr_table(gdt, ptrs)  # caution compares the update with the raw gradient
+            table = b.grad_ptr_table(gdt, ptrs)  # caution compares the update with the gradient (MARS-corrected in place, if on)
             d = _lib.HbStepDesc()
             d.param, d.param_corr = b.slab.ptr("param"), b.slab.ptr("param::ecc")
             d.grad, d.grad_ptrs = None, table.data_ptr()
-            d.exp_avg = b.slab.ptr("_update")
+            d.exp_avg, d.state_fmt = b.slab.ptr(upd_role), upd_fmt
             d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
             d.caution_count = b.caution_scratch().data_ptr() if group["caution"] else None
             d.n_chunks, d.n_tensors = n_chunks, len(b.params)
@@ -952,7 +999,10 @@ class NAdam(FirstOrder):
     _fn_name = "update_by_nadam"
     _mars_idx = 3  # ZeroGuard 0, GeneralGuard 1 (mu_product), the transform itself 2
     _init_ids = frozenset({0, 1})
-    MU_KEY = "update_by_nadam_mu_product_1"
+
+    @property
+    def MU_KEY(self) -> str:
+        return f"{self._fn()}_mu_product_1"  # scale_by_nadam_... under update_clipping
 
     def __init__(self, params, lr=0.002, betas=(0.9, 0.999), eps=1e-8, weight_decay=0, cautious_weight_decay: bool = False,
                  momentum_decay: float = 4e-3, decoupled_weight_decay: bool = False, warmup_steps=0, multi_tensor: bool = True,

@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 6
+#define HB_ABI_VERSION 7
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -62,9 +62,12 @@ enum {
 #define HB_FLAG_CAUTION 2u     /* caution mask with per-tensor rescale, heavyball/utils.py:3652-3658 */
 #define HB_FLAG_CAUTIOUS_WD 4u /* decay only where sign(p) == sign(update), heavyball/utils.py:2388 */
 #define HB_FLAG_WRITE_GRAD 8u  /* MARS: write the corrected gradient back into the gradient buffer (chainable.py:646) */
-/* The un-fused scale_by_adam / scale_by_laprop (heavyball/chainable.py:715-727, :849-862): the moments are updated and the
- * update m/denom (Adam) or m (LaProp) is WRITTEN to `param`, which is then an fp32 slab (param_fmt HB_FMT_F32) and not the
- * parameters; weight decay, learning rate and caution do not apply (hb_update_param does them afterwards). */
+/* The un-fused scale_by_adam / scale_by_laprop / scale_by_adopt / scale_by_ademamix / scale_by_nadam (heavyball/chainable.py:715-727,
+ * :849-862, :1014-1023, :820-833, :754-769): the moments are updated and the transform's update is WRITTEN as fp32 to `update_out`
+ * (an fp32 slab at the same offsets) while `param` is only read (NAdam's weight decay that is not decoupled); with `update_out`
+ * NULL the update goes to `param`, which is then that fp32 slab (param_fmt HB_FMT_F32) and not the parameters.  With 16-bit
+ * gradients the update is first rounded to their dtype, as the reference's update buffer holds it (bf16: stochastic, stream
+ * HB_STREAM_UPDATE).  Weight decay, learning rate and caution do not apply (hb_update_param does them afterwards). */
 #define HB_FLAG_UPDATE_ONLY 16u
 /* HB_ALGO_ADOPT only, its warm-up step (heavyball/chainable.py:945-946 under WarmupGuard, :587-610): exp_avg_sq <- g*g through
  * the lerp with weights (a2, one_minus_a2) = (1, 0); exp_avg and the parameters are neither read nor written. */
@@ -72,6 +75,12 @@ enum {
 /* HB_ALGO_NADAM only, weight decay that is not decoupled (heavyball/utils.py:350-379): g <- fma(p, coupled_wd, g) before the
  * moments (also the gradient caution compares with), update <- update - p * coupled_wd afterwards. */
 #define HB_FLAG_COUPLED_WD 64u
+
+/* With HB_FLAG_MARS: only the MARS prologue runs.  mars_old_grad takes the raw gradient and the corrected gradient
+ * (rounded to the gradient's dtype, heavyball/chainable.py:642-647) is WRITTEN as fp32 to `param`, which is then an fp32
+ * slab (param_fmt HB_FMT_F32) and not the parameters; the moments and the parameters are neither read nor written.  For
+ * chains that put a transform between MARS and the update (gradient clipping, heavyball/chainable.py:2694-2699). */
+#define HB_FLAG_MARS_ONLY 128u
 
 /* where the noise of stochastic rounding comes from */
 enum {
@@ -92,6 +101,7 @@ enum {
   HB_STREAM_NS_INPUT = 6, /* the legacy Newton-Schulz variant also draws from 7 for its second rounding */
   HB_STREAM_CLIP = 8,     /* bf16 stochastic rounding of a clipped bf16 gradient */
   HB_STREAM_EXP_AVG_SLOW = 9, /* AdEMAMix's slow momentum */
+  HB_STREAM_UPDATE = 10,      /* HB_FLAG_UPDATE_ONLY with bf16 gradients: the update is rounded to bf16 as the reference's update buffer is */
 };
 
 /*
@@ -145,6 +155,7 @@ typedef struct HbStepDesc {
    * (heavyball/utils.py:407-409, device array of 2*n_tensors floats); coupled_wd with HB_FLAG_COUPLED_WD */
   float coupled_wd;
   const float* tensor_scalars;
+  void* update_out; /* HB_FLAG_UPDATE_ONLY: where the update goes (fp32 slab); NULL = into `param` */
 } HbStepDesc;
 
 /* replaces fused_adam_ (heavyball/utils.py:1921-1965) / fused_laprop_ (:2247-2291) / fused_adopt_ (:2294-2315) /
@@ -166,7 +177,7 @@ int hb_fused_step_noalloc(const HbStepDesc* desc, void* stream);
 /* chain()'s non-fused tail, update_param_ (heavyball/utils.py:2393-2406): p <- p*(1 - decay*lr) + u*(-lr) on a slab,
  * with `update` an fp32 slab at the same offsets.  Uses param/param_corr/param_fmt, offsets, numel, chunks, flags
  * (CAUTION needs grad/grad_fmt and caution_count), neg_lr, one_minus_decay_lr, rng_*, and reads the update from
- * `exp_avg` (fp32). */
+ * `exp_avg`, an fp32 slab or (state_fmt == HB_FMT_BF16) a bf16 one. */
 int hb_update_param(const HbStepDesc* desc, void* stream);
 
 /* test hooks for the codec: the arithmetic of _ULPState.encode / decode (heavyball/utils.py:1296-1324) and

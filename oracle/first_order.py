@@ -142,18 +142,22 @@ def fused_laprop_(y, exp_avg, exp_avg_sq, update, grad, beta1, beta2, step, lr, 
     update_(y, u32, decay, lr, caution, cautious_decay, gp32, rounding, tidx)
 
 
-def fused_adopt_(y, update, grad, exp_avg_sq, exp_avg, beta1, beta2, step, lr, eps, decay, caution, cautious_decay, rounding, tidx):
+def fused_adopt_(y, update, grad, exp_avg_sq, exp_avg, beta1, beta2, step, lr, eps, decay, caution, cautious_decay, rounding, tidx,
+                 apply=True):  # fmt: skip
     """heavyball/utils.py:2307-2315 then :2294-2304.  ``step`` is the group's step minus one (heavyball/chainable.py:961);
-    ``eps`` stays a python float.  The update uses the second moment of the steps before; that moment is advanced last."""
+    ``eps`` stays a python float.  The update uses the second moment of the steps before; that moment is advanced last.
+    ``apply=False`` is the un-fused ``adopt`` (:2319-2334): the same moments, the update returned instead of applied."""
     beta1, beta2, lr, decay = f32(beta1), f32(beta2), lr.to(torch.float32), f32(decay)
     u32 = [promote(u) for u in update]
     g32 = [promote(g) for g in grad]
     v32 = [promote(v) for v in exp_avg_sq]
     b1 = beta_debias(beta1, step)
     m_new = lerp_(exp_avg, [u_ / ieee_sqrt(d_).clamp(min=eps) for u_, d_ in zip(u32, v32)], b1, rounding, philox.STREAM_EXP_AVG, tidx)
-    update_(y, m_new, decay, lr, caution, cautious_decay, g32, rounding, tidx)
+    if apply:
+        update_(y, m_new, decay, lr, caution, cautious_decay, g32, rounding, tidx)
     b2 = beta_debias(beta2, step + 1)
     stochastic_lerp_(exp_avg_sq, [u_ * u_ for u_ in u32], 1 - b2, rounding, philox.STREAM_EXP_AVG_SQ, tidx)
+    return m_new
 
 
 def adopt_warmup_(exp_avg_sq, update, rounding, tidx):
@@ -189,8 +193,9 @@ def linear_hl_warmup_scheduler(step: int, beta_end: float, beta_start: float, wa
 
 
 def fused_ademamix_(y, exp_avg_fast, exp_avg_slow, exp_avg_sq, update, grad, betas, step, lr, eps, decay, alpha, caution,
-                    cautious_decay, beta3_warmup, alpha_warmup, rounding, tidx):  # fmt: skip
-    """heavyball/utils.py:2135-2183 then :2086-2132.  Every scalar goes through scalar_guard here (eps too)."""
+                    cautious_decay, beta3_warmup, alpha_warmup, rounding, tidx, apply=True):  # fmt: skip
+    """heavyball/utils.py:2135-2183 then :2086-2132.  Every scalar goes through scalar_guard here (eps too).
+    ``apply=False`` is the un-fused ``ademamix_`` (:2186-2210): the update is returned instead of applied."""
     beta1, beta2, beta3_final = betas
     alpha_f = linear_warmup_scheduler(int(step), alpha_end=alpha, alpha_start=0.0, warmup=alpha_warmup)
     beta3_f = linear_hl_warmup_scheduler(int(step), beta_end=beta3_final, beta_start=beta1, warmup=beta3_warmup)
@@ -203,7 +208,9 @@ def fused_ademamix_(y, exp_avg_fast, exp_avg_slow, exp_avg_sq, update, grad, bet
     slow32 = lerp_(exp_avg_slow, u32, beta3, rounding, philox.STREAM_EXP_AVG_SLOW, tidx)
     denom = exp_avg_sq_(exp_avg_sq, u32, b2, eps, rounding, tidx)
     out = [(f_ + s_ * alpha_t) / d_ for f_, s_, d_ in zip(fast32, slow32, denom)]
-    update_(y, out, decay, lr, caution, cautious_decay, g32, rounding, tidx)
+    if apply:
+        update_(y, out, decay, lr, caution, cautious_decay, g32, rounding, tidx)
+    return out
 
 
 def nadam_moments(beta1: Tensor, step: Tensor, momentum_decay: float):
@@ -226,10 +233,12 @@ def fma_(u: Tensor, p: Tensor, alpha: float) -> Tensor:
 
 
 def fused_nadam_(param, exp_avg, exp_avg_sq, mu_product, update, grad, beta1, beta2, step, lr, eps, momentum_decay, weight_decay,
-                 decoupled_weight_decay, caution, cautious_decay, rounding, tidx):  # fmt: skip
+                 decoupled_weight_decay, caution, cautious_decay, rounding, tidx, apply=True):  # fmt: skip
     """heavyball/utils.py:2046-2083 then :2003-2043 with the helpers of :350-410.  Without ``decoupled_weight_decay`` the
     decay enters as ``weight_decay * p`` added to the gradient (and to the gradient caution compares with) and is taken
-    out of the finished update again; the parameter update itself then runs with decay 0."""
+    out of the finished update again; the parameter update itself then runs with decay 0.
+    ``apply=False`` is the un-fused ``nadam_`` (:1968-2000): the gradient that caution compares with is left alone
+    (``_nadam_prepare_weight_decay`` gets no gradient) and the update is returned instead of applied."""
     beta1_t, beta2_t, lr, eps_t = f32(beta1), f32(beta2), lr.to(torch.float32), f32(eps)
     mu, mu_next = nadam_moments(beta1_t, step, momentum_decay)
     wd = float(weight_decay)
@@ -255,7 +264,9 @@ def fused_nadam_(param, exp_avg, exp_avg_sq, mu_product, update, grad, beta1, be
         out.append(u_ / d_ * gw + e_ / d_ * ew)
     if coupled:
         out = [o_ - p_ * wd for o_, p_ in zip(out, p32)]
-    update_(param, out, f32(decay), lr, caution, cautious_decay, g32, rounding, tidx)
+    if apply:
+        update_(param, out, f32(decay), lr, caution, cautious_decay, g32, rounding, tidx)
+    return out
 
 
 def mars_correction(g: List[Tensor], old_g: List, beta1, gamma, rounding, tidx):
@@ -361,7 +372,6 @@ class FirstOrderOracle:
         beta2_scale=0.8,
     ):
         assert kind in ("adam", "laprop", "adopt", "ademamix", "nadam")
-        assert update_clipping is None or kind in ("adam", "laprop"), "update_clipping is restated for AdamW / LaProp only"
         clips = (None, "l2_clip_", "rmsnorm_clip_", "global_l2norm_clip", "global_rmsnorm_clip")
         assert gradient_clipping in clips and update_clipping in clips
         self.gradient_clipping, self.update_clipping = gradient_clipping, update_clipping
@@ -373,7 +383,7 @@ class FirstOrderOracle:
         self.momentum_decay, self.decoupled_weight_decay = momentum_decay, decoupled_weight_decay
         self.palm, self.beta2_scale = palm, beta2_scale
         if update_clipping is not None:  # heavyball/chainable.py:2676-2684: the fused transform is swapped for the un-fused one
-            self.fn_name = {"adam": "scale_by_adam", "laprop": "scale_by_laprop"}[kind]
+            self.fn_name = "scale_by_" + kind
         # constructor defaults of heavyball/__init__.py:44-80 (AdamW), :740-776 (LaProp), :640-681 (ADOPT), :124-164, :83-121
         d_lr, d_betas = {"adam": (0.0025, (0.9, 0.99)), "laprop": (0.0025, (0.9, 0.99)), "adopt": (0.0025, (0.9, 0.99)),
                          "ademamix": (0.001, (0.9, 0.999, 0.9999)), "nadam": (0.002, (0.9, 0.999))}[kind]  # fmt: skip
@@ -452,21 +462,51 @@ class FirstOrderOracle:
         m = [self._state_tensor(i, "exp_avg", grads[i].shape) for i in idx] if self.kind != "ademamix" else None
         v = [self._state_tensor(i, "exp_avg_sq", grads[i].shape) for i in idx]
         if self.update_clipping is not None:
-            # un-fused chain: scale_by_adam / scale_by_laprop (heavyball/utils.py:1852-1883, :2213-2245) -> clip -> update_param_
-            b1 = beta_debias(f32(self.betas[0]), step)
-            b2 = beta_debias(f32(self.betas[1]), step)
+            # un-fused chain (heavyball/chainable.py:2676-2701): scale_by_* leaves its result in the update buffer, which has the
+            # gradient's dtype (copy_stochastic_list_: a stochastic round for bf16, heavyball/utils.py:1868, :2229, :2000, :2209,
+            # :2327), the clip rewrites that buffer the same way (:3226-3232), update_param_ applies it (:2393-2406)
             u32 = [promote(u) for u in update]
             if self.kind == "adam":
+                b1 = beta_debias(f32(self.betas[0]), step)
+                b2 = beta_debias(f32(self.betas[1]), step)
                 ea32 = lerp_(m, u32, b1, rounding, philox.STREAM_EXP_AVG, idx)
                 denom = exp_avg_sq_(v, u32, b2, f32(self.eps), rounding, idx)
                 new = [e_ / d_ for e_, d_ in zip(ea32, denom)]
-            else:
+            elif self.kind == "laprop":
+                b1 = beta_debias(f32(self.betas[0]), step)
+                b2 = beta_debias(f32(self.betas[1]), step)
                 denom = exp_avg_sq_(v, u32, b2, f32(1e-8), rounding, idx)
                 new = lerp_(m, [u_ / d_ for u_, d_ in zip(u32, denom)], b1, rounding, philox.STREAM_EXP_AVG, idx)
+            elif self.kind == "adopt":
+                if min(self.state[i].get("_warmup_1", 0) for i in idx) < 1:  # WarmupGuard, as in the fused chain below
+                    adopt_warmup_(v, update, rounding, idx)
+                    for i in idx:
+                        self.state[i]["_warmup_1"] = self.state[i].get("_warmup_1", 0) + 1
+                    return
+                # heavyball/chainable.py:1014-1023 passes no eps: the default 1e-8 of heavyball/utils.py:2330
+                new = fused_adopt_(None, update, grad, v, m, self.betas[0], self.betas[1], step - 1, lr, 1e-8, 0.0, False, False,
+                                   rounding, idx, apply=False)  # fmt: skip
+            elif self.kind == "ademamix":
+                fast = [self._state_tensor(i, "exp_avg_fast", grads[i].shape) for i in idx]
+                slow = [self._state_tensor(i, "exp_avg_slow", grads[i].shape) for i in idx]
+                new = fused_ademamix_(None, fast, slow, v, update, grad, self.betas, step, lr, self.eps, 0.0, self.alpha, False, False,
+                                      self.beta3_warmup, self.alpha_warmup, rounding, idx, apply=False)  # fmt: skip
+            else:
+                k = self.key("mu_product")
+                for i in idx:
+                    if k not in self.state[i]:
+                        self.state[i][k] = torch.ones((), dtype=self.storage_dtype)
+                new = fused_nadam_(p, m, v, [self.state[i][k] for i in idx], update, grad, self.betas[0], self.betas[1], step, lr, self.eps,
+                                   self.momentum_decay, self.weight_decay, self.decoupled_weight_decay, False, False, rounding, idx,
+                                   apply=False)  # fmt: skip
+            for u, n, t in zip(update, new, idx):
+                copy_stochastic(u, n, rounding, philox.STREAM_UPDATE, t)
             fn = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip,
                   "global_rmsnorm_clip": global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
-            assert all(u.dtype == torch.float32 for u in update), "the oracle restates update_clipping for fp32 updates only"
-            update_param_(p, fn(new), lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)
+            for u, c, t in zip(update, fn(update), idx):
+                copy_stochastic(u, c, rounding, philox.STREAM_CLIP, t)
+            # the tail of the chain decays with the group's weight_decay whatever the transform did with it (NAdam: on top of its own)
+            update_param_(p, update, lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)
             return
         if self.kind == "adopt":
             # WarmupGuard (heavyball/chainable.py:597-610): while any tensor of this call has not had its warm-up, every

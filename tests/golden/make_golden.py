@@ -283,6 +283,24 @@ def make_palm_trajectories():
     run_traj("nadam_palm", heavyball.NAdam, dict(palm=True), shapes, torch.float32, 4)
 
 
+def make_clip_combinations():
+    """Clipping together with the switches it interacts with (heavyball/chainable.py:2676-2701): MARS runs ahead of the
+    gradient clip; with update clipping the transform is the un-fused one and the update buffer has the gradient's dtype."""
+    shapes = [(4, 8), (16,), (3, 5)]
+    A, L = heavyball.AdamW, heavyball.LaProp
+    run_traj("adamw_mars_clip_l2", A, dict(mars=True, gradient_clipping="l2_clip_", weight_decay=0.01), shapes, torch.float32, 4, grad_scale=1.0)
+    run_traj("laprop_mars_clip_global_rms_ecc_bf16grad", L, dict(mars=True, gradient_clipping="global_rmsnorm_clip", ecc="bf16+8", caution=True),
+             shapes, torch.bfloat16, 4, grad_scale=3.0)  # fmt: skip
+    run_traj("adamw_updclip_l2_bf16grad", A, dict(update_clipping="l2_clip_", weight_decay=0.01), shapes, torch.bfloat16, 4)
+    run_traj("laprop_updclip_rms_mars_bf16grad_ecc", L, dict(update_clipping="rmsnorm_clip_", mars=True, ecc="bf16+8", caution=True, lr=0.01),
+             shapes, torch.bfloat16, 4)  # fmt: skip
+    run_traj("adopt_updclip_l2", heavyball.ADOPT, dict(update_clipping="l2_clip_", weight_decay=0.01), shapes, torch.float32, 5)
+    run_traj("ademamix_updclip_global_l2_ecc", heavyball.AdEMAMix, dict(update_clipping="global_l2norm_clip", ecc="bf16+8"), shapes, torch.float32, 4)
+    run_traj("nadam_updclip_rms", heavyball.NAdam, dict(update_clipping="rmsnorm_clip_", weight_decay=0.01), shapes, torch.float32, 4)
+    run_traj("nadam_updclip_l2_decoupled_caution", heavyball.NAdam, dict(update_clipping="l2_clip_", weight_decay=0.01, decoupled_weight_decay=True,
+                                                                         caution=True), shapes, torch.float32, 4)  # fmt: skip
+
+
 def make_ns5():
     """Newton-Schulz vectors straight from the reference's functions, the bf16 stochastic round made round-half-up."""
     out = {}
@@ -379,7 +397,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "ns5", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "ns5", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -392,6 +410,8 @@ if __name__ == "__main__":
         make_variant_trajectories()
     if "palm" in which:
         make_palm_trajectories()
+    if "clipcombo" in which:
+        make_clip_combinations()
     if "ns5" in which:
         make_ns5()
     if "muon" in which:

@@ -263,15 +263,73 @@ def test_gradient_clipping_matches_oracle(kind, grad_dtype):
                 assert ((g - w).abs() <= 2.0**-7 * (w.abs() + w.abs().max())).all(), (kind, k, i, key)
 
 
+CLIP_COMBOS = [
+    # (name, class, kwargs, gradient dtype, gradient scale)
+    ("adamw_mars_gradclip_l2", "AdamW", dict(mars=True, gradient_clipping="l2_clip_", weight_decay=0.01), torch.float32, 1.0),
+    ("laprop_mars_gradclip_global_rms_ecc_caution", "LaProp", dict(mars=True, gradient_clipping="global_rmsnorm_clip", ecc="bf16+8", caution=True),
+     torch.bfloat16, 3.0),
+    ("nadam_mars_gradclip_rms_paramecc", "NAdam", dict(mars=True, gradient_clipping="rmsnorm_clip_", param_ecc="bf16+8", ecc="bf16+16"),
+     torch.float32, 2.0),
+    ("adamw_updclip_l2_bf16grad", "AdamW", dict(update_clipping="l2_clip_", weight_decay=0.01), torch.bfloat16, 1e-2),
+    ("laprop_updclip_rms_mars_ecc_caution_bf16grad", "LaProp", dict(update_clipping="rmsnorm_clip_", mars=True, ecc="bf16+8", caution=True, lr=0.01),
+     torch.bfloat16, 1e-2),
+    ("adopt_updclip_l2", "ADOPT", dict(update_clipping="l2_clip_", weight_decay=0.01), torch.float32, 1e-2),
+    ("ademamix_updclip_global_l2_ecc", "AdEMAMix", dict(update_clipping="global_l2norm_clip", ecc="bf16+8"), torch.float32, 1e-2),
+    ("nadam_updclip_rms_coupled_wd", "NAdam", dict(update_clipping="rmsnorm_clip_", weight_decay=0.01), torch.float32, 1e-2),
+    ("nadam_updclip_l2_decoupled_caution_bf16grad", "NAdam", dict(update_clipping="l2_clip_", weight_decay=0.01, decoupled_weight_decay=True,
+                                                                  caution=True), torch.bfloat16, 1e-2),
+]
+
+
+@pytest.mark.parametrize("case", CLIP_COMBOS, ids=[c[0] for c in CLIP_COMBOS])
+def test_clipping_combinations_match_oracle(case):
+    """Clipping together with the switches it interacts with (heavyball/chainable.py:2676-2701): MARS ahead of the gradient
+    clip (a pass of its own, then the step without MARS on the clipped slab); update clipping on every fused optimizer (the
+    step kernel in update-only mode, the clip, then the parameter update) and with bf16 gradients, where the update is
+    rounded to bf16 after the transform and again after the clip, as the reference's update buffer is.  The norms are
+    summed in a different order than ATen's, hence agreement to 2e-6 of each tensor's scale (bf16 updates: one ulp more
+    where the last bit of the scale moves an element across a rounding threshold)."""
+    name, cls_name, kwargs, gdt, gscale = case
+    print("case", name, flush=True)
+    cls, kind = CLS[cls_name]
+    host, params, opt, orc = H.build_pair(cls, kind, RAGGED, kwargs, DEV, rounding="philox")
+    bf16_update = gdt == torch.bfloat16 and "update_clipping" in kwargs
+    for k in range(1, 5):
+        grads = H.make_grads(RAGGED, k, gdt, gscale)
+        for p, g in zip(params, grads):
+            p.grad = g.to(DEV)
+        opt.step()
+        orc.step([g.clone() for g in grads])
+        torch.cuda.synchronize()
+        for i, p in enumerate(params):
+            st = opt.state[p][0]
+            pw = orc.params[i]
+            want = {"param": pw.primary if hasattr(pw, "primary") else pw,
+                    **{kk: v for kk, v in orc.state[i].items() if kk != "step" and isinstance(v, torch.Tensor)}}
+            got = {"param": p.data, **st}
+            if not (bf16_update or gdt == torch.bfloat16):
+                H.assert_close_in_scale(got, want, f"{name} step {k} tensor {i}")
+                continue
+            for key, w in want.items():
+                if key.endswith("::ecc") or w.dim() == 0:
+                    continue
+                ck = "param::ecc" if key == "param" else key + "::ecc"
+                g_, w_ = got[key].detach().cpu(), w
+                if ck in want:
+                    from oracle.ecc import EccTensor
+
+                    g_, w_ = EccTensor(g_, got[ck].detach().cpu()).decode(), EccTensor(w_, want[ck]).decode()
+                g_, w_ = g_.float(), w_.float()
+                off = (g_ - w_).abs() > 2e-6 * (w_.abs() + w_.abs().max()) + (2.0**-8 * w_.abs() if w.dtype != torch.float32 or ck in want else 0)
+                assert int(off.sum()) <= max(4, int(2e-3 * w_.numel())), (name, k, i, key, int(off.sum()))
+                assert ((g_ - w_).abs() <= 2.0**-6 * (w_.abs() + w_.abs().max())).all(), (name, k, i, key)
+
+
 def test_clipping_combinations_that_are_not_built_raise():
     p = [torch.nn.Parameter(torch.zeros(8, device=DEV))]
-    opt = heavyball_amd.AdamW(p, gradient_clipping="l2_clip_", mars=True)
-    p[0].grad = torch.ones(8, device=DEV)
-    with pytest.raises(NotImplementedError):
-        opt.step()
     opt = heavyball_amd.AdamW(p, update_clipping="l2_clip_")
     p[0].grad_dtype = None
-    p[0].grad = torch.ones(8, device=DEV, dtype=torch.bfloat16)  # 16-bit gradients with update_clipping are not built
+    p[0].grad = torch.ones(8, device=DEV, dtype=torch.float16)  # float16 gradients with update_clipping are not built
     with pytest.raises(NotImplementedError):
         opt.step()
     with pytest.raises(ValueError):
