@@ -73,3 +73,39 @@ def test_reference_checkpoint_loads_and_continues(path):
     opt2 = cls(params2, **kwargs)
     opt2.load_state_dict(sd)
     assert int(opt2.state[params2[0]][0]["step"]) == 3
+
+
+def test_own_checkpoints_for_the_reference_are_current(tmp_path):
+    """tests/golden/own_ckpt_*.pt are this implementation's ``state_dict()``s that tests/golden/check_own_checkpoints.py loads
+    into the reference (own_ckpt_check.json holds the outcome: every case continues to the same parameters).  They have to be
+    what the present code writes: regenerate them and compare every tensor bit for bit."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("write_own_checkpoints", os.path.join(GOLDEN, "write_own_checkpoints.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mod.main(str(tmp_path))
+    with open(os.path.join(GOLDEN, "own_ckpt_check.json")) as f:
+        checked = json.load(f)
+
+    def same(a, b, where):
+        if isinstance(a, torch.Tensor):
+            assert isinstance(b, torch.Tensor) and a.dtype == b.dtype and a.shape == b.shape, where
+            assert torch.equal(a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)), where
+        elif isinstance(a, dict):
+            assert isinstance(b, dict) and set(a) == set(b), (where, sorted(map(str, a)), sorted(map(str, b)))
+            for k in a:
+                same(a[k], b[k], f"{where}/{k}")
+        elif isinstance(a, (list, tuple)):
+            assert len(a) == len(b), where
+            for i, (x, y) in enumerate(zip(a, b)):
+                same(x, y, f"{where}[{i}]")
+        else:
+            assert a == b, (where, a, b)
+
+    for name, *_ in mod.CASES:
+        print("case", name, flush=True)
+        assert name in checked, f"{name} has not been loaded into the reference (run tests/golden/check_own_checkpoints.py)"
+        new = torch.load(os.path.join(str(tmp_path), f"own_ckpt_{name}.pt"), weights_only=True)
+        old = torch.load(os.path.join(GOLDEN, f"own_ckpt_{name}.pt"), weights_only=True)
+        same(new, old, name)
