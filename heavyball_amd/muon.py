@@ -7,7 +7,7 @@ from typing import Dict, List, Optional
 import torch
 
 from . import _lib
-from .optim import FirstOrder, HBOptimizer, _ECC_DTYPES, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, f32, lerp_weights, use_default
+from .optim import FirstOrder, HBOptimizer, _ECC_DTYPES, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, f32, lerp_weights, mars_weights, use_default
 
 #: per-iteration (a, b, c) of zeropower_via_newtonschulz5 (heavyball/utils.py:561-567)
 NS_COEFFS = (
@@ -61,12 +61,16 @@ class Muon(HBOptimizer):
         elif not nesterov:
             self._mom_mode = _lib.MOM_EMA
             self.KEY = "exp_avg_exp_avg_2"
-        if mars:
-            raise NotImplementedError("Muon: mars is not built for the Muon path")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
         self._workspace: Dict[torch.device, torch.Tensor] = {}
 
     KEY = "nesterov_ema_momentum_2"  # heavyball/chainable.py:2347-2382: update_param's walk gives the momentum guard index 2
+
+    @property
+    def _mars_idx(self) -> int:
+        """MARS' guard sits two places behind the momentum's in that walk (mars_mars_old_grad_4; _6 for MuonAdamW)."""
+        return int(self.KEY.rsplit("_", 1)[1]) + 2
+
     _mom_mode = _lib.MOM_NESTEROV_EMA
     INIT = frozenset({0, 1, 2})
 
@@ -129,6 +133,12 @@ class Muon(HBOptimizer):
             mom_prim, mom_corr = getattr(torch, group.get("storage_dtype", "float32")), None
             mom_fmt = _PLAIN_FMT[mom_prim]
 
+        mars = bool(group.get("mars"))
+        k_o = f"mars_mars_old_grad_{self._mars_idx}"
+        init_ids = set(self.INIT) | ({self._mars_idx} if mars else set())
+        if mars:
+            mars_a, mars_oma = mars_weights(group)
+
         per_bucket: Dict[int, List] = {}
         for p, g in active:
             b, i = self._find_bucket(gi, p)
@@ -142,14 +152,19 @@ class Muon(HBOptimizer):
             if mom_corr is not None:
                 b.slab.role(self.KEY + "::ecc", mom_corr)
             b.slab.role("_update", torch.float32)
+            if mars:  # stored like the momentum (zero_guard with the same group settings)
+                b.slab.role(k_o, mom_prim)
+                if mom_corr is not None:
+                    b.slab.role(k_o + "::ecc", mom_corr)
             by_dtype: Dict[torch.dtype, List] = {}
             for i, p, g in items:
                 st = self._state0(p)
-                if self.KEY not in st:
-                    st[self.KEY] = b.slab.view(self.KEY, i)
-                    if mom_corr is not None:
-                        st[self.KEY + "::ecc"] = b.slab.view(self.KEY + "::ecc", i)
-                    st.setdefault("is_initialized", set()).update(self.INIT)
+                for key in (self.KEY, k_o) if mars else (self.KEY,):
+                    if key not in st:
+                        st[key] = b.slab.view(key, i)
+                        if mom_corr is not None:
+                            st[key + "::ecc"] = b.slab.view(key + "::ecc", i)
+                        st.setdefault("is_initialized", set()).update(init_ids)
                 if self.promote and g.dtype != torch.float32:
                     g = g.float()
                 if g.dtype not in _PLAIN_FMT:
@@ -157,16 +172,22 @@ class Muon(HBOptimizer):
                 if not g.is_contiguous() or g.data_ptr() % 16 or g.device != b.device:
                     g = g.to(b.device).clone(memory_format=torch.contiguous_format)
                 by_dtype.setdefault(g.dtype, []).append((i, g))
-            if self.gradient_clipping is not None and len(by_dtype) > 1:
-                raise NotImplementedError("gradient_clipping with gradients of several dtypes in one bucket")
+            if (self.gradient_clipping is not None or mars) and len(by_dtype) > 1:
+                raise NotImplementedError("gradient_clipping / mars with gradients of several dtypes in one bucket")
             for lst in by_dtype.values():
                 lst.sort(key=lambda t: t[0])
             prepared.append((b, items, by_dtype))
         # gradient_clipping (heavyball/chainable.py:2696-2699) acts on the update before the momentum transform
         clipped = {}
-        if self.gradient_clipping is not None:
+        if self.gradient_clipping is not None or mars:
             work = [(b, lst, gdt) for b, _, by_dtype in prepared for gdt, lst in by_dtype.items()]
-            for (b, _, gdt), res in zip(work, self._clip_gradients(L, group, work, step)):
+            # MARS heads the chain (heavyball/chainable.py:2698-2699, :642-647): a pass of its own leaves the corrected gradients,
+            # rounded to the gradient dtype, in the fp32 role "_clip"; clipping and the momentum go on from there
+            for b, lst, gdt in work if mars else ():
+                if gdt not in (torch.float32, torch.bfloat16):
+                    raise NotImplementedError(f"mars with {gdt} gradients on the Muon path")
+                self._mars_prologue(L, group, b, lst, gdt, step, mars_a, mars_oma, mom_fmt, k_o)
+            for (b, _, gdt), res in zip(work, self._clip_gradients(L, group, work, step, gathered=mars)):
                 clipped[(id(b), gdt)] = res
         if self.update_clipping is not None and any(g.dtype != torch.float32 for _, g in active) and not self.promote:
             raise NotImplementedError("update_clipping with 16-bit gradients (the reference rounds the clipped update to their dtype)")
@@ -238,14 +259,17 @@ class Muon(HBOptimizer):
                     table = tables[(id(b), gdt)]
                     d = _lib.HbStepDesc()
                     d.param, d.param_corr = b.slab.ptr("param"), b.slab.ptr("param::ecc")
-                    d.grad, d.grad_ptrs = None, table.data_ptr()
+                    d.grad, d.grad_ptrs, d.grad_fmt = None, table.data_ptr(), _PLAIN_FMT[gdt]
+                    if mars:
+                        # caution compares the update with the gradient as MARS left it; a clip after MARS scales that by a
+                        # positive factor, which keeps every sign
+                        d.grad, d.grad_ptrs, d.grad_fmt = b.slab.ptr("_clip"), None, _lib.FMT_F32
                     d.exp_avg = b.slab.ptr("_update")
                     d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
                     d.caution_count = b.caution_scratch().data_ptr() if group["caution"] else None
                     d.n_chunks, d.n_tensors = n_chunks, len(b.params)
                     d.flags = flags
                     d.param_fmt = _lib.ECC_FMT[pecc] if pecc else _PLAIN_FMT[b.param_dtype]
-                    d.grad_fmt = _PLAIN_FMT[gdt]
                     d.neg_lr, d.one_minus_decay_lr = neg_lr, omdl
                     d.rng_mode, d.step, d.seed = self._rng_mode(), int(step) & 0xFFFFFFFF, self.rng_seed
                     _lib.check(L.hb_update_param(d, stream), "hb_update_param")
@@ -261,7 +285,10 @@ class MuonAdamW(Muon, FirstOrder):
     state names of the un-fused transform.  16-bit gradients on the vector route would need the extra rounding of that
     buffer and raise NotImplementedError (``promote=True`` lifts them to fp32 first).
     State names and initialisation sets follow the reference's index walk with the route in place
-    (``nesterov_ema_momentum_4`` with {2, 3, 4}; ``scale_by_adam_exp_avg_0`` / ``_exp_avg_sq_0`` with {0}).
+    (``nesterov_ema_momentum_4`` with {2, 3, 4}, ``exp_avg_exp_avg_4`` under ``nesterov=False``; ``scale_by_adam_exp_avg_0`` /
+    ``_exp_avg_sq_0`` with {0}; ``mars_mars_old_grad_6`` and a 6 in both sets under ``mars``).  ``ecc`` / ``storage_dtype`` apply
+    to the state of both routes.  ``gradient_clipping`` / ``update_clipping`` take the per-tensor kinds (``l2_clip_``,
+    ``rmsnorm_clip_``); a norm over the whole group would span the two routes and raises NotImplementedError.
     """
 
     KEY = "nesterov_ema_momentum_4"
@@ -280,8 +307,11 @@ class MuonAdamW(Muon, FirstOrder):
                          mars_gamma=mars_gamma, gradient_clipping=gradient_clipping, update_clipping=update_clipping, palm=palm,
                          beta2_scale=beta2_scale, nesterov=nesterov, compile_step=compile_step, promote=promote, ecc=ecc,
                          param_ecc=param_ecc, orig_shapes=orig_shapes, **kwargs)  # fmt: skip
-        if not nesterov or ecc or storage_dtype != "float32":
-            raise NotImplementedError("MuonAdamW: nesterov=False, ecc and non-fp32 state storage are not built")
+        if not nesterov:  # heavyball/__init__.py:527-529: exp_avg heads the matrix route instead
+            self.KEY = "exp_avg_exp_avg_4"
+        for kind in (self.gradient_clipping, self.update_clipping):
+            if kind is not None and kind.startswith("global_"):
+                raise NotImplementedError("MuonAdamW: clipping by a norm over the whole group (it would span both routes)")
         for group in self.param_groups:  # the reference's MuonAdamW has no such argument (heavyball/__init__.py:499-523)
             group.pop("heavyball_momentum", None)
         self.defaults.pop("heavyball_momentum", None)
@@ -290,8 +320,6 @@ class MuonAdamW(Muon, FirstOrder):
         return 1 if p.ndim >= 2 else 0
 
     def _run_group(self, gi, group, active):
-        if self.gradient_clipping is not None or self.update_clipping is not None:
-            raise NotImplementedError("gradient_clipping / update_clipping on the MuonAdamW path")
         matrices = [(p, g) for p, g in active if p.ndim >= 2]
         vectors = [(p, g) for p, g in active if p.ndim < 2]
         if matrices:

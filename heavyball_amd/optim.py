@@ -98,6 +98,14 @@ def lerp_weights(beta_debiased: torch.Tensor) -> Tuple[float, float]:
     return float(a), float(1 - a)
 
 
+def mars_weights(group) -> Tuple[float, float]:
+    """(a, 1 - a) of MARS' stochastic lerp.  heavyball/chainable.py:645 passes (mars_gamma, beta1) into (beta1, gamma) of
+    heavyball/utils.py:3623, so the weight is -beta1 * mars_gamma / (1 - mars_gamma)."""
+    b1m, gam = group["mars_gamma"], (group["betas"][0] if group.get("beta") is None else group["beta"])
+    am = f32(-gam * b1m / (1 - b1m))
+    return float(am), float(1 - am)
+
+
 def debiased_weights(beta: torch.Tensor, step) -> Tuple[float, float]:
     """``lerp_weights(beta_debias(beta, step))`` for an fp32 0-d ``beta``, at a fraction of the host time: the power is
     torch's own (its rounding belongs to the library), the subtractions and the division are single IEEE fp32
@@ -501,7 +509,9 @@ class HBOptimizer(torch.optim.Optimizer):
             if not gathered:  # otherwise an earlier pass (MARS) has left the gradients in the role
                 for i, g in lst:
                     b.slab.view("_clip", i).copy_(g)
-        keep = self._clip_role(L, self.gradient_clipping, "_clip", [(b, [i for i, _ in lst]) for b, lst, _ in buckets])
+        keep = None
+        if self.gradient_clipping is not None:  # None: the caller only wants the gathered role in the gradients' dtype
+            keep = self._clip_role(L, self.gradient_clipping, "_clip", [(b, [i for i, _ in lst]) for b, lst, _ in buckets])
         result = []
         for b, lst, gdt in buckets:
             role = b.slab.role("_clip", torch.float32)
@@ -708,10 +718,7 @@ class FirstOrder(HBOptimizer):
             flags |= _lib.FLAG_MARS
             if self.mars_write_grad:
                 flags |= _lib.FLAG_WRITE_GRAD
-            # heavyball/chainable.py:645 passes (mars_gamma, beta1) into (beta1, gamma) of utils.py:3623
-            b1m, gam = group["mars_gamma"], (group["betas"][0] if group.get("beta") is None else group["beta"])
-            am = f32(-gam * b1m / (1 - b1m))
-            mars_a, mars_oma = float(am), float(1 - am)
+            mars_a, mars_oma = mars_weights(group)
         else:
             mars_a, mars_oma = 0.0, 1.0
         if group["caution"]:

@@ -20,8 +20,9 @@ from typing import Dict, List, Optional
 import torch
 
 from . import _lib
-from .optim import HBOptimizer, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, debiased_weights, f32, use_default
+from .optim import HBOptimizer, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, debiased_weights, f32, mars_weights, use_default
 
+K_OLD = "mars_mars_old_grad_5"  # MARS' guard, three places behind the transform's in the reference's index walk
 K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
 
 
@@ -131,12 +132,14 @@ class SOAP(HBOptimizer):
             raise NotImplementedError("SOAP: use_precond_schedule")
         del defaults["precond_scheduler"]
         self.precond_schedule = 1 / defaults.pop("precondition_frequency")  # heavyball/__init__.py:842-858
-        if mars or ecc or param_ecc or split or precondition_1d or precond_grad_accum or storage_dtype != "float32" or not merge_dims:
-            raise NotImplementedError("SOAP on the HIP kernels: mars, ecc, param_ecc, split, precondition_1d, precond_grad_accum, "
-                                      "merge_dims=False and non-fp32 storage are not built")  # fmt: skip
+        if ecc or param_ecc or split or precond_grad_accum or storage_dtype != "float32" or not merge_dims:
+            raise NotImplementedError("SOAP on the HIP kernels: ecc, param_ecc, split, precond_grad_accum, merge_dims=False and "
+                                      "non-fp32 storage are not built")  # fmt: skip
         if palm not in (use_default, False):
             raise NotImplementedError("SOAP on the HIP kernels: palm (the beta2 schedule of heavyball/chainable.py:1921-1925) is not built")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
+        if mars and self.gradient_clipping is not None:
+            raise NotImplementedError("SOAP on the HIP kernels: mars together with gradient_clipping")
 
     def _run_group(self, gi, group, active):
         active = [(p, g) for p, g in active if p.numel() > 0]  # an empty tensor has nothing to precondition or update
@@ -168,6 +171,19 @@ class SOAP(HBOptimizer):
                 raise NotImplementedError("SOAP on the HIP kernels takes fp32 gradients (the reference rounds every intermediate of a "
                                           "16-bit update to that dtype); pass promote=True to lift them to fp32 first")  # fmt: skip
             raw[key] = [g.to(b.device, torch.float32).contiguous() for _, _, g in items]
+            if group.get("mars"):
+                # heavyball/chainable.py:642-647 heads the chain and writes the corrected gradient over the gradient itself: a
+                # pass of its own leaves it in the fp32 role "_clip", which then stands for the gradient everywhere below
+                b.slab.role(K_OLD, torch.float32)
+                for (i, p, _), g32 in zip(items, raw[key]):
+                    st = self._state0(p)
+                    if K_OLD not in st:
+                        st[K_OLD] = b.slab.view(K_OLD, i)
+                        st.setdefault("is_initialized", set()).add(5)
+                raw[key] = [g if g.data_ptr() % 16 == 0 else g.clone() for g in raw[key]]
+                lst = sorted(((i, g32) for (i, _, _), g32 in zip(items, raw[key])), key=lambda t: t[0])
+                self._mars_prologue(L, group, b, lst, torch.float32, step, *mars_weights(group), _lib.FMT_F32, K_OLD)
+                raw[key] = [b.slab.view("_clip", i) for i, _, _ in items]
         if self.gradient_clipping is not None:
             # heavyball/chainable.py:2696-2699: the clip acts on the update; the gradient itself still initialises the
             # factors (:1235-1238) and is what caution compares against
@@ -191,7 +207,7 @@ class SOAP(HBOptimizer):
                         st[K_M] = torch.zeros((1, *G.shape), dtype=torch.float32, device=b.device)
                         st[K_V] = torch.zeros((1, *G.shape), dtype=torch.float32, device=b.device)
                         GG: List[Optional[torch.Tensor]] = []
-                        if G.numel() > 1 and G.dim() >= 2:
+                        if G.numel() > 1 and (G.dim() >= 2 or group.get("precondition_1d")):  # heavyball/utils.py:1370
                             for sh in G.shape:
                                 GG.append(None if (sh > max_dim or sh == 1) else torch.zeros((1, sh, sh), dtype=torch.float32, device=b.device))
                         else:
@@ -291,9 +307,7 @@ class SOAP(HBOptimizer):
     @staticmethod
     def _update_ggt(gemm, G, GG, a: float, one_minus_a: float):
         """heavyball/utils.py:1205-1221: GG_d <- GG_d*(1-a) + (G contracted with itself over all dimensions but d)*a."""
-        if G.dim() < 2:
-            return
-        for d, m in enumerate(GG):
+        for d, m in enumerate(GG):  # a vector has a factor only under precondition_1d, a scalar never
             if m is None:
                 continue
             if d == G.dim() - 1:
@@ -318,7 +332,7 @@ class SOAP(HBOptimizer):
         main = torch.cuda.current_stream(dev)
         sides = []  # one entry per basis to refresh
         for pi, (GG, Q, exp_avg) in enumerate(jobs):
-            if exp_avg.dim() <= 2:  # bucket dimension + at most one real dimension
+            if exp_avg.dim() <= 1:  # heavyball/utils.py:837-839; a vector (bucket dimension + one) has a basis under precondition_1d
                 continue
             for d, (m, q) in enumerate(zip(GG, Q)):
                 if m is not None:

@@ -118,8 +118,9 @@ class MuonOracle:
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), weight_decay=0.0, warmup_steps=0, caution=False,
                  cautious_weight_decay=False, rounding=None, mode="newtonschulz", nesterov=True, heavyball_momentum=False,
-                 gradient_clipping=None, update_clipping=None, ecc=None, storage_dtype="float32"):  # fmt: skip
+                 gradient_clipping=None, update_clipping=None, ecc=None, storage_dtype="float32", mars=False, mars_gamma=0.0025):  # fmt: skip
         self.params = params
+        self.mars, self.mars_gamma = mars, mars_gamma
         self.ecc, self.storage_dtype = ecc, getattr(torch, storage_dtype)
         self.gradient_clipping, self.update_clipping = gradient_clipping, update_clipping
         self.nesterov, self.heavyball_momentum = nesterov, heavyball_momentum
@@ -136,6 +137,23 @@ class MuonOracle:
 
     KEY = "nesterov_ema_momentum_2"
 
+    @property
+    def MARS_KEY(self):
+        """MARS' guard comes two places behind the momentum's in the reference's index walk (heavyball/chainable.py:2347-2382):
+        mars_mars_old_grad_4 for Muon, _6 for MuonAdamW (pinned by trajectories written from the reference)."""
+        return f"mars_mars_old_grad_{int(self.KEY.rsplit('_', 1)[1]) + 2}"
+
+    def _guarded(self, i, key):
+        """zero_guard with the group's storage (heavyball/chainable.py:277-301): plain or an ECC pair."""
+        st = self.state[i]
+        if key not in st:
+            if self.ecc is None:
+                st[key] = torch.zeros_like(self.params[i], dtype=self.storage_dtype)
+            else:
+                e = EccTensor.zeros(self.params[i].shape, self.ecc)
+                st[key], st[key + "::ecc"] = e.primary, e.corr
+        return st[key] if self.ecc is None else EccTensor(st[key], st[key + "::ecc"])
+
     def step(self, grads):
         idx = [i for i, g in enumerate(grads) if g is not None]
         if not idx:
@@ -147,6 +165,13 @@ class MuonOracle:
         p = [self.params[i] for i in idx]
         grad = [grads[i] for i in idx]
         update = [g.clone() for g in grad]
+        if self.mars:  # heavyball/chainable.py:2698-2699, :642-647: first in the chain; the gradient becomes the corrected one
+            from . import first_order as fo
+
+            old = [self._guarded(i, self.MARS_KEY) for i in idx]
+            fo.mars_correction(update, old, self.mars_gamma, self.betas[0], rounding, idx)
+            for g_, u_ in zip(grad, update):
+                g_.copy_(u_)
         if self.gradient_clipping is not None:  # heavyball/chainable.py:2696-2699: on the update, ahead of the momentum
             from . import first_order as fo
 
@@ -157,16 +182,7 @@ class MuonOracle:
                     u.copy_(stochastic_round(c, rounding.noise16(philox.STREAM_CLIP, idx[j], u.shape)))
                 else:
                     u.copy_(c.to(u.dtype))
-        mom = []
-        for i in idx:  # zero_guard("momentum") with the group's storage (heavyball/chainable.py:277-301): plain or an ECC pair
-            st = self.state[i]
-            if self.KEY not in st:
-                if self.ecc is None:
-                    st[self.KEY] = torch.zeros_like(self.params[i], dtype=self.storage_dtype)
-                else:
-                    e = EccTensor.zeros(self.params[i].shape, self.ecc)
-                    st[self.KEY], st[self.KEY + "::ecc"] = e.primary, e.corr
-            mom.append(st[self.KEY] if self.ecc is None else EccTensor(st[self.KEY], st[self.KEY + "::ecc"]))
+        mom = [self._guarded(i, self.KEY) for i in idx]
         if self.heavyball_momentum:
             heavyball_momentum_(mom, update, self.betas[0], rounding, idx, self.nesterov)
         elif self.nesterov:
@@ -196,19 +212,24 @@ class MuonAdamWOracle:
     Both routes share the group's step counter and learning rate."""
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), eps=1e-8, weight_decay=0.0, warmup_steps=0, caution=False,
-                 cautious_weight_decay=False, rounding=None):  # fmt: skip
+                 cautious_weight_decay=False, rounding=None, mars=False, mars_gamma=0.0025, ecc=None, storage_dtype="float32",
+                 nesterov=True, gradient_clipping=None, update_clipping=None):  # fmt: skip
         from .first_order import FirstOrderOracle
 
+        for kind in (gradient_clipping, update_clipping):
+            assert kind in (None, "l2_clip_", "rmsnorm_clip_"), "a norm over the whole group would span both routes"
         self.params = params
         self.mat_idx = [i for i, p in enumerate(params) if p.dim() >= 2]
         self.vec_idx = [i for i, p in enumerate(params) if p.dim() < 2]
         self.rounding = rounding or HalfRounding()
         kw = dict(lr=lr, betas=betas, weight_decay=weight_decay, warmup_steps=warmup_steps, caution=caution,
-                  cautious_weight_decay=cautious_weight_decay)  # fmt: skip
-        self.muon = MuonOracle(list(params), rounding=self.rounding, **kw)
-        self.muon.KEY = "nesterov_ema_momentum_4"
+                  cautious_weight_decay=cautious_weight_decay, mars=mars, mars_gamma=mars_gamma, ecc=ecc, storage_dtype=storage_dtype,
+                  gradient_clipping=gradient_clipping, update_clipping=update_clipping)  # fmt: skip
+        self.muon = MuonOracle(list(params), rounding=self.rounding, nesterov=nesterov, **kw)
+        self.muon.KEY = "nesterov_ema_momentum_4" if nesterov else "exp_avg_exp_avg_4"
         self.adam = FirstOrderOracle("adam", list(params), eps=eps, rounding=self.rounding, **kw)
         self.adam.fn_name = "scale_by_adam"
+        self.adam.mars_idx = 6  # behind the route's guards (trajectories written from the reference)
 
     @property
     def state(self):

@@ -146,8 +146,9 @@ class SOAPOracle:
 
     def __init__(self, params, lr=3e-3, betas=(0.9, 0.95), shampoo_beta=0.95, eps=1e-8, weight_decay=0.01, precondition_frequency=2,
                  max_precond_dim=2048, precondition_1d=False, warmup_steps=0, gradient_clipping=None,
-                 update_clipping=None):  # fmt: skip
+                 update_clipping=None, mars=False, mars_gamma=0.0025):  # fmt: skip
         self.params = params
+        self.mars, self.mars_gamma = mars, mars_gamma
         self.gradient_clipping, self.update_clipping = gradient_clipping, update_clipping
         self.lr, self.betas, self.shampoo_beta, self.eps = lr, betas, shampoo_beta, eps
         self.weight_decay, self.max_precond_dim, self.precondition_1d = weight_decay, max_precond_dim, precondition_1d
@@ -158,6 +159,7 @@ class SOAPOracle:
         self.step_count = torch.zeros((), dtype=torch.int64)
         self.fired = []
 
+    K_OLD = "mars_mars_old_grad_5"  # pinned by a trajectory written from the reference
     K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
 
     def step(self, grads):
@@ -168,6 +170,14 @@ class SOAPOracle:
         lr = step_lr(self.lr, step, self.warmup_steps)
         todo_p, todo_u, todo_g = [], [], []
         updates = {i: g.clone() for i, g in enumerate(grads) if g is not None}
+        if self.mars and updates:  # heavyball/chainable.py:642-647 heads the chain; the gradient becomes the corrected one
+            from . import first_order as fo
+            from .rounding import HalfRounding
+
+            keys = list(updates)
+            old = [self.state[k].setdefault(self.K_OLD, torch.zeros_like(grads[k])) for k in keys]
+            fo.mars_correction([updates[k] for k in keys], old, self.mars_gamma, self.betas[0], HalfRounding(), keys)
+            grads = [updates[i].clone() if i in updates else None for i in range(len(grads))]
         if self.gradient_clipping is not None and updates:  # heavyball/chainable.py:2696-2699: on the update, ahead of the transform
             from . import first_order as fo
 

@@ -222,6 +222,10 @@ def run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale=1e-2, para
                         for li, lv in enumerate(v):
                             if isinstance(lv, torch.Tensor):
                                 out[f"step{k}/state{i}/{kk}/{li}"] = lv.detach().clone()
+        for i, p in enumerate(params):  # which transforms count as initialised (heavyball/chainable.py:117-133)
+            inited = flat_state(opt, p).get("is_initialized")
+            if inited is not None:
+                out[f"final/is_initialized{i}"] = torch.tensor(sorted(inited), dtype=torch.int64)
     torch.save(out, os.path.join(HERE, f"traj_{name}.pt"))
 
 
@@ -299,6 +303,27 @@ def make_clip_combinations():
     run_traj("nadam_updclip_rms", heavyball.NAdam, dict(update_clipping="rmsnorm_clip_", weight_decay=0.01), shapes, torch.float32, 4)
     run_traj("nadam_updclip_l2_decoupled_caution", heavyball.NAdam, dict(update_clipping="l2_clip_", weight_decay=0.01, decoupled_weight_decay=True,
                                                                          caution=True), shapes, torch.float32, 4)  # fmt: skip
+
+
+def make_more_switches():
+    """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
+    and ECC on MuonAdamW, SOAP's preconditioner schedule."""
+    shapes = [(8, 16), (16,), (24, 8), (4, 3, 6)]
+    run_traj("muon_mars", heavyball.Muon, dict(mars=True, weight_decay=0.01), shapes, torch.float32, 4)
+    run_traj("muon_mars_ecc_caution", heavyball.Muon, dict(mars=True, ecc="bf16+8", caution=True), shapes, torch.float32, 4)
+    run_traj("muon_mars_bf16grad", heavyball.Muon, dict(mars=True, storage_dtype="bfloat16"), shapes, torch.bfloat16, 4)
+    run_traj("muonadamw_mars_clip", heavyball.MuonAdamW, dict(mars=True, gradient_clipping="l2_clip_", weight_decay=0.01), shapes, torch.float32,
+             4, grad_scale=1.0)  # fmt: skip
+    run_traj("muonadamw_ecc_updclip", heavyball.MuonAdamW, dict(ecc="bf16+8", update_clipping="rmsnorm_clip_"), shapes, torch.float32, 4)
+    run_traj("muonadamw_plain_ema_bf16_storage", heavyball.MuonAdamW, dict(nesterov=False, storage_dtype="bfloat16"), shapes, torch.float32, 4)
+    soap_shapes = [(8, 16), (16,), (12, 6)]
+    run_traj("soap_mars", heavyball.SOAP, dict(mars=True, precondition_frequency=3), soap_shapes, torch.float32, 6)
+    # use_precond_schedule=True cannot be recorded: the reference itself fails on it (heavyball/utils.py:2411 calls .clamp on the
+    # python int that heavyball/utils.py:3497 hands it)
+    # a vector of three elements: its 3 x 3 factor has full rank by the first refresh (one outer product a step), so the refreshed
+    # basis is determined by the data and not by the rounding noise that fills the null space of a rank-deficient factor
+    run_traj("soap_precondition_1d", heavyball.SOAP, dict(precondition_1d=True, precondition_frequency=3), [(8, 16), (3,), (12, 6)],
+             torch.float32, 6)  # fmt: skip
 
 
 def make_ns5():
@@ -397,7 +422,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "ns5", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "switches", "ns5", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -412,6 +437,8 @@ if __name__ == "__main__":
         make_palm_trajectories()
     if "clipcombo" in which:
         make_clip_combinations()
+    if "switches" in which:
+        make_more_switches()
     if "ns5" in which:
         make_ns5()
     if "muon" in which:

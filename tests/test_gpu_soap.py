@@ -351,6 +351,13 @@ def test_soap_matches_reference_trajectories():
                     gk = f"step{k}/state{i}/scale_by_soap_GG_3/{li}"
                     if gk in d:
                         assert torch.allclose(opt.state[p][0]["scale_by_soap_GG_3"][li].cpu(), d[gk], rtol=1e-4, atol=1e-8)
+                ok = f"step{k}/state{i}/mars_mars_old_grad_5"
+                if ok in d:  # MARS keeps the raw gradient of the step before: a copy
+                    assert torch.equal(opt.state[p][0]["mars_mars_old_grad_5"].cpu(), d[ok])
+                assert (ok in d) == ("mars_mars_old_grad_5" in opt.state[p][0])
+        for i, p in enumerate(params):
+            if f"final/is_initialized{i}" in d:
+                assert opt.state[p][0]["is_initialized"] == set(d[f"final/is_initialized{i}"].tolist())
 
 
 def test_soap_and_muon_step_over_empty_scalar_and_degenerate_tensors():

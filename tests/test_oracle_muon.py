@@ -77,8 +77,11 @@ def test_muon_trajectory_matches_reference(path):
     for k in range(1, d["meta/steps"] + 1):
         orc.step([d[f"step{k}/g{i}"].clone() for i in range(n)])
         for i in range(n):
-            mom = d[f"step{k}/state{i}/{orc.KEY}"]
-            assert torch.equal(orc.state[i][orc.KEY], mom)  # elementwise fp32: exact
+            prefix = f"step{k}/state{i}/"
+            want_state = {kk[len(prefix):]: d[kk] for kk in d if kk.startswith(prefix) and not kk.endswith("/step")}
+            assert set(want_state) == set(orc.state[i]), (i, set(want_state), set(orc.state[i]))
+            for kk, vv in want_state.items():
+                assert torch.equal(orc.state[i][kk], vv), (k, i, kk)  # elementwise fp32: exact
             want, got = d[f"step{k}/p{i}"], orc.params[i]
             if want.dim() < 2:
                 assert torch.equal(got, want)
@@ -113,6 +116,7 @@ def test_muonadamw_trajectory_matches_reference(path):
             if want.dim() < 2:
                 H.assert_close_to_reference({"param": got, **orc.state[i]}, {"param": want, **want_state}, f"step {k} vector {i}")
             else:
-                assert torch.equal(orc.state[i]["nesterov_ema_momentum_4"], want_state["nesterov_ema_momentum_4"])
+                for kk, vv in want_state.items():
+                    assert torch.equal(orc.state[i][kk], vv), (k, i, kk)
                 prev = d[f"step{k - 1}/p{i}"] if k > 1 else d[f"init/p{i}"]
                 assert rel_fro(got - prev, want - prev) < 2e-2
