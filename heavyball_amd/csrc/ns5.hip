@@ -273,28 +273,51 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
 
   // epilogue: accumulator register r of tile (i, j) holds row (r/4)*8 + (lane/32)*4 + r%4, column lane%32
   const int erow = (lane >> 5) * 4, lcol = lane & 31;
+  // Transposed copies (X^T, the mirror of a symmetric tile).  A lane holds 4 + 4 + 4 + 4 rows of one column, lane + 32 the
+  // rows between them; v_permlane32_swap trades halves so that a lane below 32 ends up with rows 0..15 of its column and
+  // its partner with rows 16..31, 32 contiguous bytes of the transposed matrix each (64 per column) instead of 8.
+  auto store_transposed = [&](uint16_t* base, int ld, int col, int row_tile, const uint32_t (&v)[16]) {
+    uint32_t pk[4][2], out[8];
+#pragma unroll
+    for (int rb4 = 0; rb4 < 4; ++rb4) {
+      pk[rb4][0] = v[rb4 * 4 + 0] | (v[rb4 * 4 + 1] << 16);
+      pk[rb4][1] = v[rb4 * 4 + 2] | (v[rb4 * 4 + 3] << 16);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)  // h = 0: rows 0-7 | 16-23, h = 1: rows 8-15 | 24-31
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(pk[h][w], pk[h + 2][w], false, false);
+        out[h * 4 + w] = sw[0];      // rows +0..3 of the octet
+        out[h * 4 + 2 + w] = sw[1];  // rows +4..7
+      }
+    uint4* dst = reinterpret_cast<uint4*>(base + (size_t)col * ld + row_tile + (lane >> 5) * 16);
+    dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
+    dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
+  };
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int col = col0 + wn * WTN + j * 32 + lcol;
+      const int row_tile = row0 + wm * WTM + i * 32;
+      uint32_t prim[16], sec[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int row = row_tile + (q >> 2) * 8 + erow + (q & 3);
+        uint32_t h = f32_to_bf16_rne(acc[i][j][q]);
+        if (MODE == kModeS) {
+          uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * grp.mul_c);       // heavyball/utils.py:569
+          if (row == col) y = f32_to_bf16_rne(bf16_to_f32(y) + grp.diag);  // :570
+          sec[q] = y;
+        } else if (MODE == kModeY2) {
+          if (row == col) h = f32_to_bf16_rne(bf16_to_f32(h) + grp.diag);  // :572
+        }
+        prim[q] = h;
+      }
 #pragma unroll
       for (int rb4 = 0; rb4 < 4; ++rb4) {
-        const int row = row0 + wm * WTM + i * 32 + rb4 * 8 + erow;
-        uint32_t prim[4], sec[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float v = acc[i][j][rb4 * 4 + r];
-          uint32_t h = f32_to_bf16_rne(v);
-          if (MODE == kModeS) {
-            uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * grp.mul_c);           // heavyball/utils.py:569
-            if (row + r == col) y = f32_to_bf16_rne(bf16_to_f32(y) + grp.diag);  // :570
-            sec[r] = y;
-          } else if (MODE == kModeY2) {
-            if (row + r == col) h = f32_to_bf16_rne(bf16_to_f32(h) + grp.diag);  // :572
-          }
-          prim[r] = h;
-        }
+        const int row = row_tile + rb4 * 8 + erow;
         if (MODE == kModeFinal || MODE == kModePartial) {
           float o[4];
 #pragma unroll
@@ -302,7 +325,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
             if (MODE == kModePartial) {
               o[r] = acc[i][j][rb4 * 4 + r];  // one K chunk of a split product: summed and rounded by ns_split_reduce_kernel
             } else {
-              o[r] = bf16_to_f32(prim[r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
+              o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
               if (grp.round_out) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
             }
           }
@@ -323,23 +346,19 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
           }
         } else {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) g.C[(size_t)(row + r) * g.ldc + col] = (uint16_t)prim[r];
+          for (int r = 0; r < 4; ++r) g.C[(size_t)(row + r) * g.ldc + col] = (uint16_t)prim[rb4 * 4 + r];
           if (MODE == kModeS) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) g.C2[(size_t)(row + r) * g.ldc2 + col] = (uint16_t)sec[r];
-          }
-          if (MODE == kModeX) {  // transposed copy: 4 consecutive rows are 8 contiguous bytes of X^T's row `col`
-            uint2 t = make_uint2(prim[0] | (prim[1] << 16), prim[2] | (prim[3] << 16));
-            *reinterpret_cast<uint2*>(g.C2 + (size_t)col * g.ldc2 + row) = t;
-          }
-          // Symmetric modes: a tile above the diagonal is also written transposed to its place below it.  Diagonal tiles
-          // are computed in full, so a matrix that fits one tile gets the plain product.
-          if (SYMMETRIC && bi != bj) {
-            *reinterpret_cast<uint2*>(g.C + (size_t)col * g.ldc + row) = make_uint2(prim[0] | (prim[1] << 16), prim[2] | (prim[3] << 16));
-            if (MODE == kModeS)
-              *reinterpret_cast<uint2*>(g.C2 + (size_t)col * g.ldc2 + row) = make_uint2(sec[0] | (sec[1] << 16), sec[2] | (sec[3] << 16));
+            for (int r = 0; r < 4; ++r) g.C2[(size_t)(row + r) * g.ldc2 + col] = (uint16_t)sec[rb4 * 4 + r];
           }
         }
+      }
+      if constexpr (MODE == kModeX) store_transposed(g.C2, g.ldc2, col, row_tile, prim);  // X^T, the B operand of the next iteration
+      // Symmetric modes: a tile above the diagonal is also written transposed to its place below it.  Diagonal tiles
+      // are computed in full, so a matrix that fits one tile gets the plain product.
+      if (SYMMETRIC && bi != bj) {
+        store_transposed(g.C, g.ldc, col, row_tile, prim);
+        if constexpr (MODE == kModeS) store_transposed(g.C2, g.ldc2, col, row_tile, sec);
       }
     }
   }
