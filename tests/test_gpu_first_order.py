@@ -138,6 +138,47 @@ def test_bf16_params_plain():
         H.run_steps(opt, orc, params, shapes, 3, torch.bfloat16, 1e-2, DEV, tag="bf16 params " + rounding)
 
 
+@pytest.mark.parametrize("mars", [False, True], ids=["plain", "mars"])
+@pytest.mark.parametrize("rounding", ["half", "philox"])
+def test_caution_count_on_updates_that_nearly_cancel(mars, rounding):
+    """Caution's count pass decides most signs from the bf16 primaries of exp_avg (and of MARS' old gradient) and loads the
+    int8 corrections only where they could matter.  Gradients built from the oracle's own state put every element next to
+    the two decisions that can go either way: exp_avg*(1-a1) + g*a1 within +-2^-6 of zero (the corrections reach 2^-9 of
+    exp_avg), and the MARS-corrected gradient within +-2^-6 of zero.  The step must stay bit-identical to the oracle's:
+    one miscounted element changes the rescale of the whole tensor."""
+    from oracle.ecc import EccTensor
+
+    shapes = [(8192 + 24,), (96, 130), (5000,)]
+    kwargs = dict(caution=True, ecc="bf16+8", param_ecc="bf16+8", mars=mars)
+    host, params, opt, orc = H.build_pair(heavyball_amd.AdamW, "adam", shapes, kwargs, DEV, rounding=rounding)
+    H.run_steps(opt, orc, params, shapes, 2, torch.bfloat16, 1e-3, DEV, tag="ordinary steps")
+    gen = torch.Generator().manual_seed(5)
+    for k in (3, 4, 5):
+        a1 = (1 - 0.9) / (1 - 0.9**k)  # 1 - beta_debias(beta1, step)
+        c = 0.0025 * 0.9 / (1 - 0.9)  # MARS: g + c * (g - old_g), heavyball/utils.py:3623-3627 as chainable.py:645 calls it
+        grads = []
+        for i, sh in enumerate(shapes):
+            st = orc.state[i]
+            key = next(kk for kk in st if kk.endswith("exp_avg_0"))
+            m = EccTensor(st[key], st[key + "::ecc"]).decode()
+            eps = (torch.rand(sh, generator=gen) * 2 - 1) * 2.0**-6
+            target = -m * ((1 - a1) / a1) * (1 + eps)  # the (corrected) gradient that nearly cancels exp_avg
+            if mars:
+                ok = next(kk for kk in st if "old_grad" in kk and not kk.endswith("::ecc"))
+                og = EccTensor(st[ok], st[ok + "::ecc"]).decode()
+                g = (target + c * og) / (1 + c)
+                zero_gc = og * (c / (1 + c)) * (1 + eps)  # ... and, on a third of the elements, one whose correction nearly cancels itself
+                g = torch.where(torch.rand(sh, generator=gen) < 1 / 3, zero_gc, g)
+            else:
+                g = target
+            grads.append(g.to(torch.bfloat16))
+        for p_, g_ in zip(params, grads):
+            p_.grad = g_.to(DEV)
+        opt.step()
+        orc.step([g_.clone() for g_ in grads])
+        H.compare(opt, orc, params, f"nearly cancelling step {k}")
+
+
 def test_c1_full_size():
     """Benchmark configuration 1 at its full size: 4 fp32 tensors, 9,438,208 elements, 10 steps, bit-exact against the oracle."""
     shapes = [(1024, 1024), (1024,), (4096, 1024), (1024, 4096)]
