@@ -540,7 +540,7 @@ class HBOptimizer(torch.optim.Optimizer):
             for k in [k for k in g if k.startswith("_")]:
                 del g[k]
         sd["heavyball"] = {  # heavyball/utils.py:1527-1538
-            "inner_group": self.inner_group,
+            "inner_group": dict(self.inner_group),  # a snapshot: the live dict keeps counting
             "use_ema": self.use_ema,
             "ema_decay": self.ema_decay,
             "compile_step": self.compile_step,
@@ -559,6 +559,8 @@ class HBOptimizer(torch.optim.Optimizer):
                 continue
             if k == "precond_schedule":
                 v = _Unpickle(io.BytesIO(v)).load()
+            if k == "inner_group":
+                v = dict(v)  # not the caller's object: two optimizers loaded from one checkpoint must not share a counter
             setattr(self, k, v)
         sd = {k: v for k, v in state_dict.items() if k != "heavyball"}
         super().load_state_dict(sd)

@@ -20,7 +20,7 @@ from typing import Dict, List, Optional
 import torch
 
 from . import _lib
-from .optim import HBOptimizer, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, debiased_weights, f32, mars_weights, use_default
+from .optim import HBOptimizer, _ECC_DTYPES, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, debiased_weights, f32, mars_weights, use_default
 
 K_OLD = "mars_mars_old_grad_5"  # MARS' guard, three places behind the transform's in the reference's index walk
 K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
@@ -132,9 +132,11 @@ class SOAP(HBOptimizer):
             raise NotImplementedError("SOAP: use_precond_schedule")
         del defaults["precond_scheduler"]
         self.precond_schedule = 1 / defaults.pop("precondition_frequency")  # heavyball/__init__.py:842-858
-        if ecc or param_ecc or split or precond_grad_accum or storage_dtype != "float32" or not merge_dims:
-            raise NotImplementedError("SOAP on the HIP kernels: ecc, param_ecc, split, precond_grad_accum, merge_dims=False and "
-                                      "non-fp32 storage are not built")  # fmt: skip
+        # precond_grad_accum is read by PSGD's guard only (heavyball/chainable.py:304-345): SOAP's chain ignores it, and so does this
+        if split or not merge_dims:
+            raise NotImplementedError("SOAP on the HIP kernels: split and merge_dims=False are not built")
+        if mars and (ecc or storage_dtype != "float32"):
+            raise NotImplementedError("SOAP on the HIP kernels: mars together with ecc or non-fp32 storage")
         if palm not in (use_default, False):
             raise NotImplementedError("SOAP on the HIP kernels: palm (the beta2 schedule of heavyball/chainable.py:1921-1925) is not built")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
@@ -155,6 +157,13 @@ class SOAP(HBOptimizer):
         omdl, neg_lr = float(1 - decay * lr), float(-lr)
         flags = (_lib.FLAG_CAUTION if group["caution"] else 0) | (_lib.FLAG_CAUTIOUS_WD if group.get("cautious_weight_decay", False) else 0)
         is_precond = bool(group["is_preconditioning"])
+        pecc = group.get("param_ecc")
+        if group.get("ecc"):
+            mom_prim, mom_corr = _ECC_DTYPES[group["ecc"]]
+            mom_fmt = _lib.ECC_FMT[group["ecc"]]
+        else:
+            mom_prim, mom_corr = getattr(torch, group.get("storage_dtype", "float32")), None
+            mom_fmt = _PLAIN_FMT[mom_prim]
 
         per_bucket: Dict[int, List] = {}
         for p, g in active:
@@ -165,8 +174,8 @@ class SOAP(HBOptimizer):
             if b.device.type != "cuda":
                 raise _lib.HbError("the optimizer step runs on the GPU only: parameters must live on a CUDA/HIP device")
             self._check_home(b, items)
-            if b.param_dtype != torch.float32:
-                raise NotImplementedError("SOAP on the HIP kernels takes fp32 parameters")
+            if b.param_dtype != torch.float32 and not group.get("param_ecc"):
+                raise NotImplementedError("SOAP on the HIP kernels takes fp32 parameters (or param_ecc)")
             if any(g.dtype != torch.float32 for _, _, g in items) and not self.promote:
                 raise NotImplementedError("SOAP on the HIP kernels takes fp32 gradients (the reference rounds every intermediate of a "
                                           "16-bit update to that dtype); pass promote=True to lift them to fp32 first")  # fmt: skip
@@ -204,8 +213,10 @@ class SOAP(HBOptimizer):
                     G = b.slab.view("_clip", i).reshape(G0.shape) if self.gradient_clipping is not None else G0  # the update
                     st = self._state0(p)
                     if K_M not in st:  # first step: initialise, no update (heavyball/chainable.py:372-377, utils.py:1362-1388)
-                        st[K_M] = torch.zeros((1, *G.shape), dtype=torch.float32, device=b.device)
-                        st[K_V] = torch.zeros((1, *G.shape), dtype=torch.float32, device=b.device)
+                        for km in (K_M, K_V):  # zero_guard with the group's storage (heavyball/chainable.py:277-301)
+                            st[km] = torch.zeros((1, *G.shape), dtype=mom_prim, device=b.device)
+                            if mom_corr is not None:
+                                st[km + "::ecc"] = torch.zeros((1, *G.shape), dtype=mom_corr, device=b.device)
                         GG: List[Optional[torch.Tensor]] = []
                         if G.numel() > 1 and (G.dim() >= 2 or group.get("precondition_1d")):  # heavyball/utils.py:1370
                             for sh in G.shape:
@@ -236,19 +247,33 @@ class SOAP(HBOptimizer):
                     a2, oma2 = debiased_weights(beta2, adam_step)
                     if gp is G:
                         gp = G.clone()
-                    _lib.check(L.hb_adam_precond(st[K_M].data_ptr(), st[K_V].data_ptr(), gp.data_ptr(), gp.data_ptr(), gp.numel(), a1, oma1,
+                    # moments kept as bf16 or as an ECC pair are widened to fp32 for the step and written back through the
+                    # codec; the update comes from the fp32 values before that rounding, as in the reference (utils.py:1842-1849)
+                    m32, v32 = self._widen(L, st, K_M, mom_fmt, stream), self._widen(L, st, K_V, mom_fmt, stream)
+                    _lib.check(L.hb_adam_precond(m32.data_ptr(), v32.data_ptr(), gp.data_ptr(), gp.data_ptr(), gp.numel(), a1, oma1,
                                                  a2, oma2, float(f32(group["eps"])), stream), "hb_adam_precond")  # fmt: skip
-                    back = self._project(gemm, gp, Q, back=True)
-                    out.copy_(back)
+                    if mom_fmt != _lib.FMT_F32:
+                        base = int(b.slab.offsets_np[i])
+                        self._narrow(L, st, K_M, m32, mom_fmt, _lib.STREAM_EXP_AVG, step, base, stream)
+                        self._narrow(L, st, K_V, v32, mom_fmt, _lib.STREAM_EXP_AVG_SQ, step, base, stream)
+                    back = self._project(gemm, gp, Q, back=True, out=out)
+                    if back is not out:  # no basis at all, or the last product went through a moved dimension
+                        out.copy_(back)
                     sb = beta_debias(group["shampoo_beta"], step)  # heavyball/chainable.py:1244: python float and int64 0-d tensor
                     a = 1 - sb
                     a = a.to(torch.float32) if isinstance(a, torch.Tensor) else f32(a)
                     self._update_ggt(gemm, G, GG, float(a), float(1 - a))
                     if is_precond:
-                        refresh.append((GG, Q, st[K_M]))
+                        if mom_fmt == _lib.FMT_F32:
+                            refresh.append((GG, Q, st[K_M]))
+                        else:  # the rotation reads exp_avg as stored (heavyball/utils.py:883) and writes it back through the codec
+                            refresh.append((GG, Q, self._widen(L, st, K_M, mom_fmt, stream), st, int(b.slab.offsets_np[i])))
                     updated.append(i)
                 if refresh:
                     self._refresh(gemm, refresh)
+                    for job in refresh:
+                        if len(job) > 3:
+                            self._narrow(L, job[3], K_M, job[2], mom_fmt, _lib.STREAM_SOAP_ROTATE, step, job[4], stream)
             if updated:
                 pending.append((b, sorted(updated), items, keep))
         if self.update_clipping is not None and pending:  # heavyball/chainable.py:2700-2701
@@ -260,7 +285,7 @@ class SOAP(HBOptimizer):
                 offsets, numel = b.slab.meta()
                 chunks, n_chunks = b.slab.chunks(tuple(updated))
                 d = _lib.HbStepDesc()
-                d.param = b.slab.ptr("param")
+                d.param, d.param_corr = b.slab.ptr("param"), b.slab.ptr("param::ecc")
                 ptrs = [0] * len(b.params)
                 for (i, _, _), g32 in zip(items, keep):
                     ptrs[i] = g32.data_ptr()
@@ -270,24 +295,59 @@ class SOAP(HBOptimizer):
                 d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
                 d.caution_count = b.caution_scratch().data_ptr() if group["caution"] else None
                 d.n_chunks, d.n_tensors = n_chunks, len(b.params)
-                d.flags, d.param_fmt, d.grad_fmt = flags, _PLAIN_FMT[b.param_dtype], _lib.FMT_F32
+                d.flags, d.param_fmt, d.grad_fmt = flags, (_lib.ECC_FMT[pecc] if pecc else _PLAIN_FMT[b.param_dtype]), _lib.FMT_F32
                 d.neg_lr, d.one_minus_decay_lr = neg_lr, omdl
                 d.rng_mode, d.step, d.seed = self._rng_mode(), int(step) & 0xFFFFFFFF, self.rng_seed
                 _lib.check(L.hb_update_param(d, current_stream_ptr(b.device)), "hb_update_param")
         self._last_launch = (None, [k for *_, k in pending], clip_keep)
 
+    def _rehome_state(self):
+        """torch's ``load_state_dict`` casts floating-point state to the parameter's dtype: the moments go back to their storage
+        dtype (their values are representable there, heavyball/chainable.py:2452-2484 does the same)."""
+        super()._rehome_state()
+        for group in self.param_groups:
+            for p in group["params"]:
+                st = self.state.get(p, {}).get(0) if p in self.state else None
+                if not isinstance(st, dict):
+                    continue
+                for key in (K_M, K_V, K_M + "::ecc", K_V + "::ecc"):
+                    if isinstance(st.get(key), torch.Tensor):
+                        st[key] = st[key].to(self._role_dtype(group, key)).contiguous()
+
     # -- pieces ----------------------------------------------------------------------------------------------------
+    def _widen(self, L, st, key, fmt, stream):
+        """The moment ``st[key]`` as fp32: itself when stored so, else a decoded copy."""
+        t = st[key]
+        if fmt == _lib.FMT_F32:
+            return t
+        if fmt == _lib.FMT_BF16:
+            return t.float()
+        out = torch.empty(t.shape, dtype=torch.float32, device=t.device)
+        _lib.check(L.hb_ecc_decode(t.data_ptr(), st[key + "::ecc"].data_ptr(), out.data_ptr(), t.numel(), fmt, stream), "hb_ecc_decode")
+        return out
+
+    def _narrow(self, L, st, key, value, fmt, stream_id, step, base, stream):
+        """``copy_stochastic_`` of an fp32 moment into its bf16 or ECC storage (heavyball/utils.py:2363-2370, :1296-1311); the noise
+        of element e is that of flat index ``base + e``, ``base`` being the parameter's offset in its slab."""
+        t = st[key]
+        if fmt == _lib.FMT_BF16:
+            _lib.check(L.hb_sr_bf16(value.data_ptr(), t.data_ptr(), t.numel(), self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF,
+                                    stream_id, base, stream), "hb_sr_bf16")  # fmt: skip
+        else:
+            _lib.check(L.hb_ecc_encode(value.data_ptr(), t.data_ptr(), st[key + "::ecc"].data_ptr(), t.numel(), fmt, self._rng_mode(),
+                                       self.rng_seed, int(step) & 0xFFFFFFFF, stream_id, base, stream), "hb_ecc_encode")  # fmt: skip
+
     @staticmethod
-    def _mode_product(gemm, X, q, d: int, back: bool):
+    def _mode_product(gemm, X, q, d: int, back: bool, out=None):
         """Contracts dimension ``d`` of X with the square matrix q: out[.., j, ..] = sum_i X[.., i, ..] q[i, j]
         (q[j, i] when ``back``). The first and last dimension are plain GEMMs on a reshaped view; a middle one is
-        moved to the front first."""
+        moved to the front first.  ``out`` (contiguous, X's shape) receives the result of a first- or last-dimension product."""
         if d == 0:
-            Y = torch.empty_like(X)
+            Y = torch.empty_like(X) if out is None else out
             gemm(q, X.reshape(X.shape[0], -1), Y.view(X.shape[0], -1), ta=not back)
             return Y
         if d == X.dim() - 1:
-            Y = torch.empty_like(X)
+            Y = torch.empty_like(X) if out is None else out
             gemm(X.reshape(-1, X.shape[-1]), q, Y.view(-1, X.shape[-1]), tb=back)
             return Y
         Xp = X.movedim(d, 0).contiguous()
@@ -296,12 +356,15 @@ class SOAP(HBOptimizer):
         return Y.movedim(0, d).contiguous()
 
     @classmethod
-    def _project(cls, gemm, X, Q, back: bool):
-        """heavyball/utils.py:1391-1411: every dimension that has a basis is rotated by it (by its transpose when ``back``)."""
+    def _project(cls, gemm, X, Q, back: bool, out=None):
+        """heavyball/utils.py:1391-1411: every dimension that has a basis is rotated by it (by its transpose when ``back``).
+        The last product writes into ``out`` where it can (a first or last dimension); the caller copies otherwise."""
         cur = X
+        last = max((d for d, q in enumerate(Q) if q is not None), default=-1)
         for d, q in enumerate(Q):
             if q is not None:
-                cur = cls._mode_product(gemm, cur, q[0], d, back)
+                direct = out is not None and d == last and d in (0, X.dim() - 1)
+                cur = cls._mode_product(gemm, cur, q[0], d, back, out if direct else None)
         return cur
 
     @staticmethod
@@ -331,7 +394,7 @@ class SOAP(HBOptimizer):
         dev = gemm.device
         main = torch.cuda.current_stream(dev)
         sides = []  # one entry per basis to refresh
-        for pi, (GG, Q, exp_avg) in enumerate(jobs):
+        for pi, (GG, Q, exp_avg, *_) in enumerate(jobs):
             if exp_avg.dim() <= 1:  # heavyball/utils.py:837-839; a vector (bucket dimension + one) has a basis under precondition_1d
                 continue
             for d, (m, q) in enumerate(zip(GG, Q)):

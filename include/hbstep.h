@@ -102,6 +102,7 @@ enum {
   HB_STREAM_CLIP = 8,     /* bf16 stochastic rounding of a clipped bf16 gradient */
   HB_STREAM_EXP_AVG_SLOW = 9, /* AdEMAMix's slow momentum */
   HB_STREAM_UPDATE = 10,      /* HB_FLAG_UPDATE_ONLY with bf16 gradients: the update is rounded to bf16 as the reference's update buffer is */
+  HB_STREAM_SOAP_ROTATE = 11, /* SOAP: exp_avg written back to bf16 / ECC storage after its rotation into a refreshed basis */
 };
 
 /*
@@ -180,8 +181,9 @@ int hb_fused_step_noalloc(const HbStepDesc* desc, void* stream);
  * `exp_avg`, an fp32 slab or (state_fmt == HB_FMT_BF16) a bf16 one. */
 int hb_update_param(const HbStepDesc* desc, void* stream);
 
-/* test hooks for the codec: the arithmetic of _ULPState.encode / decode (heavyball/utils.py:1296-1324) and
- * stochastic_round_ (:2341-2355) on n contiguous elements starting at flat index `flat_base` of stream `stream_id` */
+/* the codec on its own: the arithmetic of _ULPState.encode / decode (heavyball/utils.py:1296-1324) and
+ * stochastic_round_ (:2341-2355) on n contiguous elements starting at flat index `flat_base` of stream `stream_id`.
+ * Used by the tests of the codec, by param_ecc at construction and by SOAP's moments when they are stored narrow. */
 int hb_ecc_encode(const float* src, void* primary, void* corr, int64_t n, int32_t fmt, int32_t rng_mode, uint64_t seed,
                   uint32_t step, uint32_t stream_id, int64_t flat_base, void* stream);
 int hb_ecc_decode(const void* primary, const void* corr, float* dst, int64_t n, int32_t fmt, void* stream);

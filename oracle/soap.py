@@ -100,21 +100,31 @@ def project(grad: Tensor, Q: List[Optional[Tensor]], back: bool) -> Tensor:
     return grad
 
 
-def adam_(exp_avg: Tensor, exp_avg_sq: Tensor, grad: Tensor, beta1, beta2, step: Tensor, eps) -> Tensor:
-    """heavyball/utils.py:1852-1883 on fp32 state: returns exp_avg / max(sqrt(exp_avg_sq), eps) after the moment updates."""
+def adam_(exp_avg, exp_avg_sq, grad: Tensor, beta1, beta2, step: Tensor, eps, rounding=None, tidx=0) -> Tensor:
+    """heavyball/utils.py:1852-1883: returns exp_avg / max(sqrt(exp_avg_sq), eps) from the moments as computed in fp32, BEFORE
+    they are written back to their storage (fp32: the same values; bf16 or an ECC pair: rounded on the way, :1842-1849)."""
+    from . import first_order as fo
+    from . import philox
+    from .rounding import HalfRounding
+
+    rounding = rounding or HalfRounding()
     beta1, beta2, eps = f32(beta1), f32(beta2), f32(eps)
     b1 = beta_debias(beta1, step)
     b2 = beta_debias(beta2, step)
-    a1 = 1 - b1
-    exp_avg.copy_(exp_avg * (1 - a1) + grad * a1)
-    a2 = 1 - b2
-    exp_avg_sq.copy_(exp_avg_sq * (1 - a2) + (grad * grad) * a2)
-    denom = ieee_sqrt(exp_avg_sq).clamp(min=eps)
-    return exp_avg / denom
+    exp_avg32 = fo.lerp_([exp_avg], [grad], b1, rounding, philox.STREAM_EXP_AVG, [tidx])[0]
+    denom = fo.exp_avg_sq_([exp_avg_sq], [grad], b2, eps, rounding, [tidx])[0]
+    return exp_avg32 / denom
 
 
-def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg: Tensor):
-    """heavyball/utils.py:829-900 (heavy=False): one power-iteration step + QR per side, then rotate exp_avg into the new basis."""
+def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg, rounding=None, tidx=0):
+    """heavyball/utils.py:829-900 (heavy=False): one power-iteration step + QR per side, then rotate exp_avg into the new basis
+    (decoded to fp32 for the rotation and written back through copy_stochastic_, :883-884)."""
+    from . import first_order as fo
+    from . import philox
+    from .rounding import HalfRounding
+
+    stored = exp_avg
+    exp_avg = fo.promote(stored)
     if exp_avg.dim() <= 1:
         return
     new_qs = []
@@ -135,7 +145,8 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
     to_sh = ",".join([f"...{i}{o}" for m, i, o in zip(new_qs, in_str.upper(), out_str) if m is not None])
     out_lin = "".join([o if o in to_sh else i for i, o in zip(in_str, out_str)])
     subs = f"...{in_str},{from_sh},{to_sh}->...{out_lin}"
-    exp_avg.copy_(torch.einsum(subs, exp_avg, *[q for q in Q if q is not None], *[q for q in new_qs if q is not None]))
+    rotated = torch.einsum(subs, exp_avg, *[q for q in Q if q is not None], *[q for q in new_qs if q is not None])
+    fo.copy_stochastic(stored, rotated, rounding or HalfRounding(), philox.STREAM_SOAP_ROTATE, tidx)
     for q, qn in zip(Q, new_qs):
         if q is not None:
             q.copy_(qn)
@@ -146,18 +157,51 @@ class SOAPOracle:
 
     def __init__(self, params, lr=3e-3, betas=(0.9, 0.95), shampoo_beta=0.95, eps=1e-8, weight_decay=0.01, precondition_frequency=2,
                  max_precond_dim=2048, precondition_1d=False, warmup_steps=0, gradient_clipping=None,
-                 update_clipping=None, mars=False, mars_gamma=0.0025):  # fmt: skip
-        self.params = params
+                 update_clipping=None, mars=False, mars_gamma=0.0025, ecc=None, storage_dtype="float32", param_ecc=None,
+                 caution=False, cautious_weight_decay=False, precond_grad_accum=False, rounding=None):  # fmt: skip
+        from . import philox
+        from .ecc import MODES, EccTensor
+        from .rounding import HalfRounding
+
+        # precond_grad_accum is read by PSGD's guard only (heavyball/chainable.py:304-345): SOAP's chain ignores it
+        self.rounding = rounding or HalfRounding()
+        self.ecc, self.storage_dtype = ecc, getattr(torch, storage_dtype)
+        self.caution, self.cautious_weight_decay = caution, cautious_weight_decay
+        self.param_ecc = param_ecc
         self.mars, self.mars_gamma = mars, mars_gamma
+        self._state_init = [dict() for _ in params]
+        if param_ecc is not None:  # heavyball/chainable.py:2421-2444: the live parameter is narrowed at construction
+            narrowed = []
+            for i, p in enumerate(params):
+                pd, cd = MODES[param_ecc]
+                e = EccTensor(p.to(pd), torch.zeros(p.shape, dtype=cd))
+                if p.dtype != pd:
+                    e.compute_correction(p.float(), self.rounding.at_step(0).uniform(philox.STREAM_INIT_PARAM, i, p.shape))
+                narrowed.append(e)
+                self._state_init[i]["param::ecc"] = e.corr
+            params = narrowed
+        self.params = params
         self.gradient_clipping, self.update_clipping = gradient_clipping, update_clipping
         self.lr, self.betas, self.shampoo_beta, self.eps = lr, betas, shampoo_beta, eps
         self.weight_decay, self.max_precond_dim, self.precondition_1d = weight_decay, max_precond_dim, precondition_1d
         self.warmup_steps = warmup_steps
         self.schedule = 1 / precondition_frequency
         self.inner_group = {}
-        self.state = [dict() for _ in params]
+        self.state = self._state_init
         self.step_count = torch.zeros((), dtype=torch.int64)
         self.fired = []
+
+    def _moment(self, st, key, like):
+        """zero_guard with the group's storage (heavyball/chainable.py:277-301)."""
+        from .ecc import EccTensor
+
+        if key not in st:
+            if self.ecc is None:
+                st[key] = torch.zeros_like(like, dtype=self.storage_dtype)
+            else:
+                e = EccTensor.zeros(like.shape, self.ecc)
+                st[key], st[key + "::ecc"] = e.primary, e.corr
+        return st[key] if self.ecc is None else EccTensor(st[key], st[key + "::ecc"])
 
     K_OLD = "mars_mars_old_grad_5"  # pinned by a trajectory written from the reference
     K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
@@ -168,7 +212,7 @@ class SOAPOracle:
         step = self.step_count
         self.fired.append(bool(is_precond))
         lr = step_lr(self.lr, step, self.warmup_steps)
-        todo_p, todo_u, todo_g = [], [], []
+        todo_p, todo_u, todo_g, todo_i = [], [], [], []
         updates = {i: g.clone() for i, g in enumerate(grads) if g is not None}
         if self.mars and updates:  # heavyball/chainable.py:642-647 heads the chain; the gradient becomes the corrected one
             from . import first_order as fo
@@ -192,23 +236,26 @@ class SOAPOracle:
             st = self.state[i]
             u = updates[i].reshape(merged_shape(g.shape, self.max_precond_dim)).unsqueeze(0)  # merged view + the bucket dimension
             if self.K_M not in st:  # first step: ZeroGuard + GeneralGuard init, no update (heavyball/chainable.py:372-377)
-                st[self.K_M] = torch.zeros_like(u)
-                st[self.K_V] = torch.zeros_like(u)
+                self._moment(st, self.K_M, u)
+                self._moment(st, self.K_V, u)
                 # heavyball/chainable.py:1235-1238: the initial factors come from the gradient, not from the (clipped) update
                 g0 = g.clone().reshape(merged_shape(g.shape, self.max_precond_dim)).unsqueeze(0)
                 st[self.K_GG], st[self.K_Q] = init_preconditioner(g0, self.max_precond_dim, self.precondition_1d)
                 continue
             Q, GG = st[self.K_Q], st[self.K_GG]
             gp = project(u, Q, False)
-            precond = adam_(st[self.K_M], st[self.K_V], gp, self.betas[0], self.betas[1], step - 1, self.eps)
+            rounding = self.rounding.at_step(int(step))
+            m_st, v_st = self._moment(st, self.K_M, u), self._moment(st, self.K_V, u)
+            precond = adam_(m_st, v_st, gp, self.betas[0], self.betas[1], step - 1, self.eps, rounding, i)
             precond = project(precond, Q, True)
             beta = beta_debias(self.shampoo_beta, step)  # heavyball/chainable.py:1244
             update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta)
             if is_precond:
-                refresh_basis(GG, Q, st[self.K_M])
+                refresh_basis(GG, Q, m_st, rounding, i)
             todo_p.append(p)
             todo_u.append(precond.squeeze(0).reshape(p.shape))
             todo_g.append(g)
+            todo_i.append(i)
         if todo_p and self.update_clipping is not None:  # heavyball/chainable.py:2700-2701
             from . import first_order as fo
 
@@ -216,4 +263,5 @@ class SOAPOracle:
                   "global_rmsnorm_clip": fo.global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
             todo_u = fn(todo_u)
         if todo_p:
-            update_param_(todo_p, todo_u, lr, self.weight_decay, False, False, todo_g)
+            update_param_(todo_p, todo_u, lr, self.weight_decay, self.caution, self.cautious_weight_decay, todo_g,
+                          self.rounding.at_step(int(step)), todo_i)

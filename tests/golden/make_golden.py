@@ -324,6 +324,17 @@ def make_more_switches():
     # basis is determined by the data and not by the rounding noise that fills the null space of a rank-deficient factor
     run_traj("soap_precondition_1d", heavyball.SOAP, dict(precondition_1d=True, precondition_frequency=3), [(8, 16), (3,), (12, 6)],
              torch.float32, 6)  # fmt: skip
+    # switches of SOAP that act outside the preconditioner (the parameter's storage) or on its moments' storage; a combination the
+    # reference itself cannot run is reported and leaves no fixture
+    for name, kw in [("soap_param_ecc_caution", dict(param_ecc="bf16+8", caution=True, precondition_frequency=3)),
+                     ("soap_ecc", dict(ecc="bf16+8", precondition_frequency=3)),
+                     ("soap_bf16_storage", dict(storage_dtype="bfloat16", precondition_frequency=3)),
+                     ("soap_split", dict(split=True, max_precond_dim=8, precondition_frequency=3)),
+                     ("soap_precond_grad_accum", dict(precond_grad_accum=True, precondition_frequency=3))]:  # fmt: skip
+        try:
+            run_traj(name, heavyball.SOAP, kw, soap_shapes, torch.float32, 6)
+        except Exception as exc:  # noqa: BLE001
+            print(f"{name}: the reference fails with {type(exc).__name__}: {str(exc)[:200]}")
 
 
 def make_ns5():

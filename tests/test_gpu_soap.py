@@ -7,6 +7,8 @@ import json
 import os
 
 import pytest
+
+from oracle.ecc import EccTensor
 import torch
 
 import heavyball_amd
@@ -336,6 +338,8 @@ def test_soap_matches_reference_trajectories():
         kwargs = json.loads(d["meta/kwargs"])
         n = len([k for k in d if k.startswith("init/p")])
         params = [torch.nn.Parameter(d[f"init/p{i}"].clone().to(DEV)) for i in range(n)]
+        for p in params:
+            p.grad_dtype = None  # param_ecc narrows the parameter, the gradients stay fp32
         opt = heavyball_amd.SOAP(params, **kwargs)
         for k in range(1, d["meta/steps"] + 1):
             for i, p in enumerate(params):
@@ -345,8 +349,18 @@ def test_soap_matches_reference_trajectories():
             if k == 1:
                 _adopt_basis(opt, params, lambda i, li: d[f"step1/state{i}/scale_by_soap_Q_3/{li}"].to(DEV))
             for i, p in enumerate(params):
-                want = d[f"step{k}/p{i}"]
-                assert torch.allclose(p.detach().cpu(), want, rtol=1e-3, atol=2e-6), (k, i, (p.detach().cpu() - want).abs().max())
+                want, got = d[f"step{k}/p{i}"], p.detach().cpu()
+                ck = f"step{k}/state{i}/param::ecc"
+                if ck in d:  # param_ecc: the decoded pair
+                    want, got = EccTensor(want, d[ck]).decode(), EccTensor(got, opt.state[p][0]["param::ecc"].cpu()).decode()
+                # moments kept in plain bf16: a product summed in another order can land on the other side of a bf16 rounding, which
+                # moves that entry of the update by 2^-8 of itself, i.e. the parameter by lr * 2^-8 per step
+                atol = 5e-5 if "bf16_storage" in path else 2e-6
+                assert got.dtype == want.dtype and torch.allclose(got, want, rtol=1e-3, atol=atol), (k, i, (got - want).abs().max())
+                for km in ("scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2"):  # storage of the moments
+                    ref, have = d[f"step{k}/state{i}/{km}"], opt.state[p][0][km]
+                    assert have.dtype == ref.dtype and tuple(have.shape) == tuple(ref.shape)
+                    assert (f"step{k}/state{i}/{km}::ecc" in d) == (km + "::ecc" in opt.state[p][0])
                 for li in range(3):
                     gk = f"step{k}/state{i}/scale_by_soap_GG_3/{li}"
                     if gk in d:
@@ -358,6 +372,77 @@ def test_soap_matches_reference_trajectories():
         for i, p in enumerate(params):
             if f"final/is_initialized{i}" in d:
                 assert opt.state[p][0]["is_initialized"] == set(d[f"final/is_initialized{i}"].tolist())
+
+
+@pytest.mark.parametrize("rounding", ["half", "philox"])
+@pytest.mark.parametrize("kwargs", [dict(ecc="bf16+8"), dict(storage_dtype="bfloat16"), dict(ecc="fp16+16", param_ecc="bf16+8", caution=True)],
+                         ids=["ecc", "bf16_storage", "ecc16_param_ecc_caution"])
+def test_soap_narrow_storage_matches_oracle(kwargs, rounding):
+    """exp_avg / exp_avg_sq kept as bf16 or as an ECC pair, and the parameter as an ECC pair: widened for the step, written
+    back through the codec (after the rotation of a basis refresh too), with the oracle's noise (round-half-up, and Philox
+    indexed by the parameter's offset in its slab).  Square gradients, so both sides' own eigh give the same basis up to
+    signs; products are summed in another order than the oracle's, so decoded values agree to a tolerance (the step to
+    5e-3, a moment to that plus one unit of its storage)."""
+    from oracle.rounding import HalfRounding, PhiloxRounding
+
+    shapes = [(40, 40), (24, 24)]
+    host, params = H.make_params(shapes, DEV, scale=0.5)
+    opt = heavyball_amd.SOAP(params, precondition_frequency=3, **kwargs)
+    opt.rounding, opt.rng_seed = rounding, 11
+    if kwargs.get("param_ecc"):
+        for b in opt._buckets[0]:
+            for i, p in enumerate(b.params):
+                j = [id(q) for q in params].index(id(p))
+                opt._encode_param(b, i, host[j].to(DEV).contiguous(), opt.param_groups[0])
+    base = opt._buckets[0][0].slab.offsets_np.tolist()
+    r = HalfRounding() if rounding == "half" else PhiloxRounding(11, base=base)
+    orc = osoap.SOAPOracle([h.clone() for h in host], precondition_frequency=3, rounding=r, **kwargs)
+
+    def value(t, corr):
+        t = t.detach().cpu()
+        return EccTensor(t, corr.detach().cpu()).decode() if corr is not None else t.float()
+
+    unit = {"bf16+8": 2.0**-8 / 127, "fp16+16": 2.0**-11 / 32767}.get(kwargs.get("ecc"), 2.0**-8)  # of the value's magnitude
+    for k in range(1, 8):
+        grads = H.make_grads(shapes, k, torch.float32, 1e-2)
+        prev = [value(p.data, opt.state[p][0].get("param::ecc") if p in opt.state else None) for p in params]
+        prev_o = [value(q.primary, q.corr) if isinstance(q, EccTensor) else q.clone() for q in orc.params]
+        for p, g in zip(params, grads):
+            p.grad = g.to(DEV)
+        opt.step()
+        orc.step([g.clone() for g in grads])
+        torch.cuda.synchronize()
+        for i, p in enumerate(params):
+            st, so = opt.state[p][0], orc.state[i]
+            q = orc.params[i]
+            got = value(p.data, st.get("param::ecc")) - prev[i]
+            want = (value(q.primary, q.corr) if isinstance(q, EccTensor) else q) - prev_o[i]
+            if k == 1:
+                assert torch.equal(got, torch.zeros_like(got))
+                continue
+            # a parameter kept as an ECC pair moves in units of 2^-8/127 of a bf16 ulp: compare the step to that resolution too
+            slack = 4 * (2.0**-8 / 127) * prev[i].abs().max().item() * prev[i].numel() ** 0.5 if kwargs.get("param_ecc") else 0.0
+            assert (got - want).norm().item() <= 5e-3 * want.norm().item() + slack, (k, i, rel_fro(got, want))
+            for km in (orc.K_M, orc.K_V):
+                have, ref = value(st[km], st.get(km + "::ecc")), value(so[km], so.get(km + "::ecc"))
+                assert st[km].dtype == so[km].dtype
+                fix = torch.abs if km == orc.K_M else (lambda t: t)  # eigenvector signs are free
+                assert ((fix(have) - fix(ref)).abs() <= 5e-3 * ref.abs().max() + 2 * unit * ref.abs()).all(), (k, i, km)
+    if not kwargs.get("param_ecc"):  # a checkpoint carries the narrow moments: a second optimizer continues bit for bit
+        params2 = [torch.nn.Parameter(p.detach().clone()) for p in params]
+        opt2 = heavyball_amd.SOAP(params2, precondition_frequency=3, **kwargs)
+        opt2.rounding, opt2.rng_seed = rounding, 11
+        opt2.load_state_dict(opt.state_dict())
+        grads = H.make_grads(shapes, 8, torch.float32, 1e-2)
+        for o, ps in ((opt, params), (opt2, params2)):
+            for p, g in zip(ps, grads):
+                p.grad = g.to(DEV)
+            o.step()
+        torch.cuda.synchronize()
+        for p, p2 in zip(params, params2):
+            assert torch.equal(p.detach(), p2.detach())
+            for km in (orc.K_M, orc.K_V):
+                assert torch.equal(opt.state[p][0][km], opt2.state[p2][0][km])
 
 
 def test_soap_and_muon_step_over_empty_scalar_and_degenerate_tensors():

@@ -6,6 +6,8 @@ import json
 import os
 
 import pytest
+
+from oracle.ecc import EccTensor
 import torch
 
 from oracle import soap
@@ -69,11 +71,17 @@ def test_soap_trajectory_matches_reference(path):
     for k in range(1, d["meta/steps"] + 1):
         orc.step([d[f"step{k}/g{i}"].clone() for i in range(n)])
         for i in range(n):
-            want = d[f"step{k}/p{i}"]
-            assert torch.allclose(orc.params[i], want, rtol=1e-4, atol=1e-6), (k, i, (orc.params[i] - want).abs().max())
+            want, got = d[f"step{k}/p{i}"], orc.params[i]
+            if isinstance(got, EccTensor):  # param_ecc: compare the decoded value, the pair's resolution is 2^-8 of a bf16 ulp
+                want, got = EccTensor(want, d[f"step{k}/state{i}/param::ecc"]).decode(), got.decode()
+            assert torch.allclose(got, want, rtol=1e-4, atol=1e-6), (k, i, (got - want).abs().max())
             for key in (orc.K_M, orc.K_V):
-                assert tuple(orc.state[i][key].shape) == tuple(d[f"step{k}/state{i}/{key}"].shape)
-                assert torch.allclose(orc.state[i][key], d[f"step{k}/state{i}/{key}"], rtol=1e-3, atol=1e-6), (k, i, key)
+                have, ref = orc.state[i][key], d[f"step{k}/state{i}/{key}"]
+                assert tuple(have.shape) == tuple(ref.shape) and have.dtype == ref.dtype
+                if key + "::ecc" in orc.state[i]:
+                    have, ref = EccTensor(have, orc.state[i][key + "::ecc"]).decode(), EccTensor(ref, d[f"step{k}/state{i}/{key}::ecc"]).decode()
+                tol = 1e-2 if have.dtype == torch.bfloat16 else 1e-3  # plain bf16 storage: one ulp is 2^-8
+                assert torch.allclose(have.float(), ref.float(), rtol=tol, atol=1e-6), (k, i, key)
             for li, gg in enumerate(orc.state[i][orc.K_GG]):
                 gk = f"step{k}/state{i}/{orc.K_GG}/{li}"
                 assert (gg is None) == (gk not in d)
