@@ -45,6 +45,7 @@ struct Problem {
   int K, lda, ldb, ldc, ldc2, ldf;
   int f_rows, f_cols, f_transposed;  // valid extent of F (the workspace is padded to tile multiples)
   float scale;                       // ModeFinal: post-scale
+  float mul_c, diag;                 // ModeS: c and b; ModeY2: diag = a (per matrix: one launch may mix coefficient schedules)
   int tiles_m, tiles_n;              // tile grid of C
   int tile_begin;                    // first workgroup id (a multiple of 8)
   int n_tiles;                       // tiles computed: the upper triangle of the grid in the symmetric modes, else all
@@ -53,7 +54,6 @@ constexpr int kMaxGroup = 28;
 struct GroupArgs {
   Problem p[kMaxGroup];
   int n_problems;
-  float mul_c, diag;  // ModeS: c and b; ModeY2: diag = a  (the same for every matrix of the group)
   int round_out;      // ModeFinal: the reference's update buffer is bf16, so the scaled result is rounded to bf16 (to nearest)
 };
 static_assert(sizeof(GroupArgs) <= 4096, "the group travels as a kernel argument");
@@ -182,6 +182,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
   g.A = ka->p[pi].A; g.B = ka->p[pi].B; g.C = ka->p[pi].C; g.C2 = ka->p[pi].C2; g.F = ka->p[pi].F;
   g.K = ka->p[pi].K; g.lda = ka->p[pi].lda; g.ldb = ka->p[pi].ldb; g.ldc = ka->p[pi].ldc; g.ldc2 = ka->p[pi].ldc2; g.ldf = ka->p[pi].ldf;
   g.f_rows = ka->p[pi].f_rows; g.f_cols = ka->p[pi].f_cols; g.f_transposed = ka->p[pi].f_transposed; g.scale = ka->p[pi].scale;
+  g.mul_c = ka->p[pi].mul_c; g.diag = ka->p[pi].diag;
   const int row0 = bi * BM, col0 = bj * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -307,11 +308,11 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
         const int row = row_tile + (q >> 2) * 8 + erow + (q & 3);
         uint32_t h = f32_to_bf16_rne(acc[i][j][q]);
         if (MODE == kModeS) {
-          uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * grp.mul_c);       // heavyball/utils.py:569
-          if (row == col) y = f32_to_bf16_rne(bf16_to_f32(y) + grp.diag);  // :570
+          uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * g.mul_c);       // heavyball/utils.py:569
+          if (row == col) y = f32_to_bf16_rne(bf16_to_f32(y) + g.diag);  // :570
           sec[q] = y;
         } else if (MODE == kModeY2) {
-          if (row == col) h = f32_to_bf16_rne(bf16_to_f32(h) + grp.diag);  // :572
+          if (row == col) h = f32_to_bf16_rne(bf16_to_f32(h) + g.diag);  // :572
         }
         prim[q] = h;
       }
@@ -378,13 +379,13 @@ struct PrepItem {
   int rows, cols, ldx, ldxt, transpose;
   int n_blocks, block_begin;  // sum of squares: this matrix owns workgroups [block_begin, block_begin + n_blocks)
   int tiles_c, tile_begin;    // conversion: 64 x 64 tiles, tiles_c per tile row, first workgroup id
+  int legacy;                 // two stochastic rounds (legacy_zeropower_via_newtonschulz5) instead of one
 };
 constexpr int kMaxPrep = 28;
 struct PrepGroup {
   PrepItem it[kMaxPrep];
   int n_items;
   float eps;
-  int legacy;
   int bf16_update;  // the reference's update buffer is bf16: norm and quotient are bf16 values (to nearest), no stochastic round
   Rng rng;
 };
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
   const float* __restrict__ g = ka->it[pi].g;
   const int rows = ka->it[pi].rows, cols = ka->it[pi].cols, transpose = ka->it[pi].transpose;
   const int64_t flat_base = ka->it[pi].flat_base;
-  const int legacy = grp.bf16_update ? 2 : grp.legacy;  // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input)
+  const int legacy = grp.bf16_update ? 2 : ka->it[pi].legacy;  // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input)
   const Rng rng = grp.rng;
   __shared__ uint16_t tile[64][64 + 8];  // +8: rows 144 B apart, so the column reads below spread over the banks
   const float nrm = ka->it[pi].norm[0];
@@ -626,7 +627,7 @@ static int launch_group(const GroupArgs& a, int n_blocks, hipStream_t s) {
 // starts workgroups in id order, so the long tiles start first and the short ones fill in behind them) and launched
 // in groups of at most kMaxGroup.
 template <int MODE>
-static int gemm_stage(std::vector<Problem> probs, int tile, float mul_c, float diag, hipStream_t s, int round_out = 0) {
+static int gemm_stage(std::vector<Problem> probs, int tile, hipStream_t s, int round_out = 0) {
 #ifndef HB_GEMM_CFG
 #define HB_GEMM_CFG 256, 256, 64, 2, 4, 2
 #endif
@@ -635,8 +636,6 @@ static int gemm_stage(std::vector<Problem> probs, int tile, float mul_c, float d
   for (size_t first = 0; first < probs.size(); first += kMaxGroup) {
     GroupArgs a{};
     a.n_problems = (int)std::min<size_t>(kMaxGroup, probs.size() - first);
-    a.mul_c = mul_c;
-    a.diag = diag;
     a.round_out = round_out;
     int blocks = 0;
     for (int i = 0; i < a.n_problems; ++i) {
@@ -655,18 +654,24 @@ static int gemm_stage(std::vector<Problem> probs, int tile, float mul_c, float d
   return HB_OK;
 }
 
+// coeffs_host: 15 floats per matrix when per_matrix, else one table of 15; flags likewise (HB_NS_BF16_UPDATE must agree over the batch)
 static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
-                            const float* coeffs_host, int32_t legacy, float eps, const float* post_scale, int32_t rng_mode, uint64_t seed,
-                            uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes, hipStream_t s,
-                            const char* who) {
-  if (n_mats <= 0 || !g || !out || !rows || !cols || !coeffs_host || !post_scale || !flat_base || !workspace)
+                            const float* coeffs_host, const int32_t* flags, bool per_matrix, float eps, const float* post_scale,
+                            int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
+                            int64_t workspace_bytes, hipStream_t s, const char* who) {
+  if (n_mats <= 0 || !g || !out || !rows || !cols || !coeffs_host || !flags || !post_scale || !flat_base || !workspace)
     return set_error(HB_EINVAL, "%s: null pointer or empty batch", who);
   if (rng_mode != HB_RNG_HALF && rng_mode != HB_RNG_PHILOX) return set_error(HB_EINVAL, "%s: bad rng_mode", who);
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return set_error(HB_EINVAL, "%s: workspace must be 256-byte aligned", who);
-  if (legacy & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE)) return set_error(HB_EINVAL, "%s: unknown flag bits", who);
-  const int bf16_update = (legacy & HB_NS_BF16_UPDATE) != 0;
-  legacy &= HB_NS_LEGACY;
-  if (legacy && bf16_update) return set_error(HB_EINVAL, "%s: the legacy schedule on a bf16 update is not built", who);
+  auto flag_of = [&](int i) { return flags[per_matrix ? i : 0]; };
+  auto coeff_of = [&](int i, int k) { return coeffs_host[(per_matrix ? (size_t)i * 15 : 0) + k]; };
+  const int bf16_update = (flag_of(0) & HB_NS_BF16_UPDATE) != 0;
+  for (int i = 0; i < n_mats; ++i) {
+    if (flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE)) return set_error(HB_EINVAL, "%s: unknown flag bits", who);
+    if (((flag_of(i) & HB_NS_BF16_UPDATE) != 0) != (bf16_update != 0))
+      return set_error(HB_EINVAL, "%s: HB_NS_BF16_UPDATE must be set for every matrix of a call or for none", who);
+    if ((flag_of(i) & HB_NS_LEGACY) && bf16_update) return set_error(HB_EINVAL, "%s: the legacy schedule on a bf16 update is not built", who);
+  }
   for (int i = 0; i < n_mats; ++i) {
     if (!g[i] || !out[i]) return set_error(HB_EINVAL, "%s: null matrix pointer at %d", who, i);
     if (rows[i] <= 0 || cols[i] <= 0 || rows[i] > (1 << 20) || cols[i] > (1 << 20)) return set_error(HB_EINVAL, "%s: bad shape at %d", who, i);
@@ -695,7 +700,6 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
     PrepGroup pg{};
     pg.n_items = std::min(kMaxPrep, n_mats - first);
     pg.eps = eps;
-    pg.legacy = legacy;
     pg.bf16_update = bf16_update;
     pg.rng = rng;
     int blocks = 0, tiles = 0;
@@ -714,6 +718,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
       q.ldx = (int)p.np;
       q.ldxt = (int)p.mp;
       q.transpose = p.rows > p.cols;
+      q.legacy = (flag_of(i) & HB_NS_LEGACY) != 0;
       const int64_t n = p.rows * p.cols;
       q.n_blocks = (int)std::min<int64_t>(1024, (n + 4095) / 4096);
       q.block_begin = blocks;
@@ -740,7 +745,9 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
     std::vector<Problem> probs(idx.size());
     for (int it = 0; it < 5; ++it) {
       const int cur = it & 1, nxt = cur ^ 1;
-      const float ca = coeffs_host[3 * it], cb = coeffs_host[3 * it + 1], cc = coeffs_host[3 * it + 2];
+      auto ca = [&](int i) { return coeff_of(i, 3 * it); };      // the iteration's (a, b, c) of matrix i
+      auto cb = [&](int i) { return coeff_of(i, 3 * it + 1); };
+      auto cc = [&](int i) { return coeff_of(i, 3 * it + 2); };
       // S = X X^T, Y = c S + b I   (S is symmetric bit for bit: only the upper triangle of tiles is computed; a product
       // that is split along K goes through raw partial products and ns_split_reduce_kernel instead)
       std::vector<Problem> whole, chunks;
@@ -750,6 +757,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         Problem q{};
         q.tiles_m = q.tiles_n = (int)(p.mp / t);
         q.lda = (int)p.np; q.ldb = (int)p.np;
+        q.mul_c = cc(i); q.diag = cb(i);
         if (p.split == 0) {
           q.A = X(i, cur); q.B = X(i, cur); q.K = (int)p.np;
           q.C = S(i); q.ldc = (int)p.mp; q.C2 = Y(i); q.ldc2 = (int)p.mp;
@@ -766,16 +774,16 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         }
       }
       if (!whole.empty())
-        if (int rc = gemm_stage<kModeS>(whole, t, cc, cb, s)) return rc;
+        if (int rc = gemm_stage<kModeS>(whole, t, s)) return rc;
       if (!chunks.empty()) {
-        if (int rc = gemm_stage<kModePartial>(chunks, t, 0.0f, 0.0f, s)) return rc;
+        if (int rc = gemm_stage<kModePartial>(chunks, t, s)) return rc;
         for (size_t k = 0; k < idx.size(); ++k) {
           const int i = idx[k];
           const NsPlan& p = plans[i];
           if (p.split == 0) continue;
           const int64_t n = p.mp * p.mp;
           ns_split_reduce_kernel<<<(unsigned)std::min<int64_t>(1024, (n + 255) / 256), 256, 0, s>>>(
-              reinterpret_cast<const float*>(base[i] + p.off_split), p.split, (int)p.mp, S(i), Y(i), cc, cb);
+              reinterpret_cast<const float*>(base[i] + p.off_split), p.split, (int)p.mp, S(i), Y(i), cc(i), cb(i));
         }
       }
       // Y2 = Y S + a I  (S symmetric: its rows are the K-contiguous operand; Y2 is a polynomial in S, so only the
@@ -787,9 +795,10 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         q.A = Y(i); q.B = S(i); q.K = (int)p.mp; q.lda = (int)p.mp; q.ldb = (int)p.mp;
         q.C = Y2(i); q.ldc = (int)p.mp;
         q.tiles_m = q.tiles_n = (int)(p.mp / t);
+        q.diag = ca(i);
         probs[k] = q;
       }
-      if (int rc = gemm_stage<kModeY2>(probs, t, 0.0f, ca, s)) return rc;
+      if (int rc = gemm_stage<kModeY2>(probs, t, s)) return rc;
       // X = Y2 X  ==  gemm(Y2, X^T)
       for (size_t k = 0; k < idx.size(); ++k) {
         const int i = idx[k];
@@ -806,7 +815,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         }
         probs[k] = q;
       }
-      if (int rc = it < 4 ? gemm_stage<kModeX>(probs, t, 0.0f, 0.0f, s) : gemm_stage<kModeFinal>(probs, t, 0.0f, 0.0f, s, bf16_update)) return rc;
+      if (int rc = it < 4 ? gemm_stage<kModeX>(probs, t, s) : gemm_stage<kModeFinal>(probs, t, s, bf16_update)) return rc;
     }
   }
   return check_launch(who);
@@ -835,13 +844,21 @@ extern "C" int hb_ns5_batched(int32_t n_mats, const float* const* g, float* cons
                               const float* coeffs_host, int32_t legacy, float eps, const float* post_scale, int32_t rng_mode,
                               uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                               void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, coeffs_host, legacy, eps, post_scale, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, coeffs_host, &legacy, false, eps, post_scale, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched");
+}
+
+extern "C" int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
+                                    const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
+                                    uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
+                                    void* stream_) {
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, coeffs_host, flags, true, eps, post_scale, rng_mode, seed, step, flat_base,
+                              workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched_mixed");
 }
 
 extern "C" int hb_ns5(const float* g, float* out, int64_t rows, int64_t cols, const float* coeffs_host, int32_t legacy, float eps,
                       float post_scale, int32_t rng_mode, uint64_t seed, uint32_t step, int64_t flat_base, void* workspace,
                       int64_t workspace_bytes, void* stream_) {
-  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, coeffs_host, legacy, eps, &post_scale, rng_mode, seed, step, &flat_base, workspace,
+  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, coeffs_host, &legacy, false, eps, &post_scale, rng_mode, seed, step, &flat_base, workspace,
                               workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5");
 }

@@ -217,9 +217,8 @@ class Muon(HBOptimizer):
                 # orthogonalise every update with two or more dimensions (heavyball/chainable.py:1117-1126)
                 if mode not in ("newtonschulz", "legacy_newtonschulz"):
                     raise NotImplementedError(f"zeroth_power_mode={mode!r}")
-                # every matrix of the bucket goes through Newton-Schulz in grouped launches; the legacy coefficient
-                # table applies to square inputs only (heavyball/utils.py:790-795), so there are at most two batches
-                batches = {False: [], True: []}
+                # every matrix of the bucket goes through Newton-Schulz in the same grouped launches; under the legacy mode the
+                # square ones take the legacy coefficient table and input rounding (heavyball/utils.py:790-795), the others the default
                 # with bf16 gradients the reference's update buffer is bf16 and Newton-Schulz normalises it in bf16
                 gdts = set(by_dtype)
                 if gdts - {torch.float32, torch.bfloat16} or len(gdts) > 1:
@@ -227,25 +226,28 @@ class Muon(HBOptimizer):
                 ns_flags = _lib.NS_BF16_UPDATE if gdts == {torch.bfloat16} else 0
                 if ns_flags and mode == "legacy_newtonschulz":
                     raise NotImplementedError("Muon: the legacy Newton-Schulz schedule with bfloat16 gradients")
+                mats = []
                 for i, p, _ in items:
                     if p.dim() < 2:
                         continue
                     rows, cols = p.shape[0], p.numel() // p.shape[0]
-                    batches[mode == "legacy_newtonschulz" and rows == cols].append((i, rows, cols))
-                for legacy, mats in batches.items():
-                    arr = (ctypes.c_float * 15)(*ns_coefficients(LEGACY_COEFFS if legacy else NS_COEFFS))
-                    for part in self._ns_parts(L, mats):
-                        n = len(part)
-                        rows_a = (ctypes.c_int64 * n)(*[r for _, r, _ in part])
-                        cols_a = (ctypes.c_int64 * n)(*[c for _, _, c in part])
-                        ptrs = (ctypes.c_void_p * n)(*[b.slab.view("_update", i).data_ptr() for i, _, _ in part])
-                        scale = (ctypes.c_float * n)(*[max(1, r / c) ** 0.5 for _, r, c in part])  # heavyball/utils.py:808-809
-                        base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
-                        nbytes = ctypes.c_int64()
-                        _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows_a, cols_a, ctypes.byref(nbytes)))
-                        ws = self._ws(b.device, nbytes.value)
-                        _lib.check(L.hb_ns5_batched(n, ptrs, ptrs, rows_a, cols_a, arr, ns_flags | int(legacy), 1e-7, scale, self._rng_mode(), self.rng_seed,
-                                                    int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream), "hb_ns5_batched")  # fmt: skip
+                    mats.append((i, rows, cols))
+                coeff_tables = {False: ns_coefficients(NS_COEFFS), True: ns_coefficients(LEGACY_COEFFS)}
+                for part in self._ns_parts(L, mats):
+                    n = len(part)
+                    legacy = [mode == "legacy_newtonschulz" and r == c for _, r, c in part]
+                    rows_a = (ctypes.c_int64 * n)(*[r for _, r, _ in part])
+                    cols_a = (ctypes.c_int64 * n)(*[c for _, _, c in part])
+                    ptrs = (ctypes.c_void_p * n)(*[b.slab.view("_update", i).data_ptr() for i, _, _ in part])
+                    scale = (ctypes.c_float * n)(*[max(1, r / c) ** 0.5 for _, r, c in part])  # heavyball/utils.py:808-809
+                    base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
+                    arr = (ctypes.c_float * (15 * n))(*[x for lg in legacy for x in coeff_tables[lg]])
+                    flag_a = (ctypes.c_int32 * n)(*[ns_flags | int(lg) for lg in legacy])
+                    nbytes = ctypes.c_int64()
+                    _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows_a, cols_a, ctypes.byref(nbytes)))
+                    ws = self._ws(b.device, nbytes.value)
+                    _lib.check(L.hb_ns5_batched_mixed(n, ptrs, ptrs, rows_a, cols_a, arr, flag_a, 1e-7, scale, self._rng_mode(), self.rng_seed,
+                                                      int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream), "hb_ns5_batched_mixed")  # fmt: skip
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group
             keep.append(self._clip_updates(L, [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared]))
         for b, items, by_dtype in prepared:

@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 7
+#define HB_ABI_VERSION 8
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -259,6 +259,14 @@ int hb_ns5_batched_workspace_bytes(int32_t n_mats, const int64_t* rows, const in
 int hb_ns5_batched(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                    const float* coeffs_host, int32_t legacy, float eps, const float* post_scale, int32_t rng_mode, uint64_t seed,
                    uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes, void* stream);
+/* hb_ns5_batched with a coefficient table and a flag word per matrix (coeffs_host: n_mats x 15 floats, flags: n_mats
+ * words, both in HOST memory): under zeroth_power_mode = "legacy_newtonschulz" the dispatcher gives square matrices the
+ * legacy variant and the others the default one (heavyball/utils.py:790-795), and one call still covers the whole group.
+ * HB_NS_BF16_UPDATE must be set for all matrices or for none.  Bit-identical to separate calls per schedule. */
+int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
+                         const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
+                         uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
+                         void* stream);
 
 /*
  * SOAP.  hb_gemm_f32: C[M,N] = op(A) op(B) in fp32 on the matrix cores; op(A) = A^T when trans_a (A given as [K,M]),

@@ -81,6 +81,42 @@ def test_ns5_batched_equals_one_by_one():
         assert rel_fro(alone, muon.orthogonal(G.clone(), PhiloxRounding(5, step=3, base=[bases[k]]), 0)) < NS_TOL
 
 
+def test_ns5_mixed_schedules_in_one_call_equal_one_call_per_matrix():
+    """hb_ns5_batched_mixed: a coefficient table and a flag word per matrix.  Under the legacy mode the square matrices take
+    the legacy table and its two input roundings, the others the default one (heavyball/utils.py:790-795); one grouped call
+    over all of them gives, bit for bit, what a call per matrix gives, in both tile classes and with a K-split product."""
+    shapes = [(1024, 1024), (1024, 1280), (300, 300), (130, 515), (2304, 2048), (64, 64), (200, 8500), (1280, 1280)]
+    gen = torch.Generator().manual_seed(12)
+    Gs = [torch.randn(s, generator=gen) * 1e-2 for s in shapes]
+    legacy = [r == c for r, c in shapes]
+    assert any(legacy) and not all(legacy)
+    bases = [4096 * 8 * k for k in range(len(shapes))]
+    L = _lib.lib()
+    n = len(Gs)
+    rows = (ctypes.c_int64 * n)(*[g.shape[0] for g in Gs])
+    cols = (ctypes.c_int64 * n)(*[g.shape[1] for g in Gs])
+    nbytes = ctypes.c_int64()
+    _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows, cols, ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
+    gs = [g.to(DEV).contiguous() for g in Gs]
+    outs = [torch.empty_like(g) for g in gs]
+    tabs = {False: ns_coeff_array(muon.NS_COEFFS), True: ns_coeff_array(muon.LEGACY_COEFFS)}
+    arr = (ctypes.c_float * (15 * n))(*[x for lg in legacy for x in tabs[lg]])
+    flags = (ctypes.c_int32 * n)(*[int(lg) for lg in legacy])
+    gp = (ctypes.c_void_p * n)(*[g.data_ptr() for g in gs])
+    op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    scale = (ctypes.c_float * n)(*[max(1, g.shape[0] / g.shape[1]) ** 0.5 for g in Gs])
+    base = (ctypes.c_int64 * n)(*bases)
+    _lib.check(L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None))
+    torch.cuda.synchronize()
+    for k, G in enumerate(Gs):
+        print("case", tuple(G.shape), "legacy" if legacy[k] else "default", flush=True)
+        alone = run_ns5(G, legacy=legacy[k], rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=bases[k])
+        assert torch.equal(outs[k].cpu().view(torch.int32), alone.view(torch.int32)), f"matrix {k} {tuple(G.shape)}"
+    flags[1] |= 2  # HB_NS_BF16_UPDATE on one matrix only: refused
+    assert L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None) != 0
+
+
 def test_ns5_mirrored_symmetric_products():
     """Only the upper triangle of tiles of X X^T and of Y S is computed and mirrored; the output has to be what the full
     products give within the Newton-Schulz tolerance on matrices with off-diagonal tiles in both tile classes."""
