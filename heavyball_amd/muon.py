@@ -284,8 +284,9 @@ class MuonAdamW(Muon, FirstOrder):
 
     The un-fused ``scale_by_adam`` writes its result into the update buffer, which has the gradient's dtype; for fp32
     gradients that is the same arithmetic as the fused Adam step, so the vectors run on ``hb_fused_step`` under the
-    state names of the un-fused transform.  16-bit gradients on the vector route would need the extra rounding of that
-    buffer and raise NotImplementedError (``promote=True`` lifts them to fp32 first).
+    state names of the un-fused transform.  bf16 gradients on the vector route take the step kernel's update-only mode,
+    which rounds the update to bf16 as that buffer does, and ``hb_update_param`` after it; fp16 gradients raise
+    NotImplementedError (``promote=True`` lifts them to fp32 first).
     State names and initialisation sets follow the reference's index walk with the route in place
     (``nesterov_ema_momentum_4`` with {2, 3, 4}, ``exp_avg_exp_avg_4`` under ``nesterov=False``; ``scale_by_adam_exp_avg_0`` /
     ``_exp_avg_sq_0`` with {0}; ``mars_mars_old_grad_6`` and a 6 in both sets under ``mars``).  ``ecc`` / ``storage_dtype`` apply
@@ -297,6 +298,7 @@ class MuonAdamW(Muon, FirstOrder):
     INIT = frozenset({2, 3, 4})
     _algo = _lib.ALGO_ADAM
     _fn_name = "scale_by_adam"
+    _unfused_for_narrow_grads = True
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), eps=1e-8, weight_decay=0, cautious_weight_decay: bool = False,
                  warmup_steps=0, multi_tensor: bool = True, storage_dtype: str = "float32", mars: bool = False,
@@ -327,9 +329,6 @@ class MuonAdamW(Muon, FirstOrder):
         if matrices:
             Muon._run_group(self, gi, group, matrices)
         if vectors:
-            if any(g.dtype != torch.float32 for _, g in vectors) and not self.promote:
-                raise NotImplementedError("MuonAdamW: 16-bit gradients on the Adam route (the un-fused transform rounds its result "
-                                          "to the gradient's dtype); pass promote=True or fp32 gradients")  # fmt: skip
             FirstOrder._run_group(self, gi, group, vectors)
 
 

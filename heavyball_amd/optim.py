@@ -700,10 +700,15 @@ class FirstOrder(HBOptimizer):
         """Per-bucket descriptor fields beyond the common ones; returns what must stay alive until the stream is done."""
         return None
 
+    #: take the un-fused form of the transform (scale_by_*, then update_param_) whenever a gradient is narrower than fp32: the
+    #: reference's un-fused transform leaves its result in an update buffer of the gradient's dtype (MuonAdamW's vector route)
+    _unfused_for_narrow_grads = False
+
     def _run_group(self, gi, group, active):
-        unfused = self.update_clipping is not None
+        narrow = not self.promote and any(g.dtype != torch.float32 for _, g in active)
+        unfused = self.update_clipping is not None or (self._unfused_for_narrow_grads and narrow)
         if unfused and any(g.dtype == torch.float16 for _, g in active) and not self.promote:
-            raise NotImplementedError("update_clipping with float16 gradients (the clipped update is re-rounded to bfloat16 or kept in float32)")
+            raise NotImplementedError("the un-fused chain (update_clipping, MuonAdamW's vector route) with float16 gradients")
         L = _lib.lib()
         step = group["step"]
         lr = f32(group["lr"])
@@ -833,7 +838,7 @@ class FirstOrder(HBOptimizer):
             self._last_launch = (d, (table, chunks, offsets, numel, clip, extra))  # kept for profiling harnesses
         if not unfused:
             return
-        keep = self._clip_updates(L, [(b, [i for i, _ in lst]) for b, lst, _ in work])
+        keep = self._clip_updates(L, [(b, [i for i, _ in lst]) for b, lst, _ in work]) if self.update_clipping is not None else None
         decay_py = group["weight_decay"]  # update_param_ keeps decay a python float (heavyball/utils.py:2393-2406)
         for b, lst, gdt in work:
             upd_role, upd_fmt = "_update", _lib.FMT_F32

@@ -394,6 +394,7 @@ class FirstOrderOracle:
         self.storage_dtype = getattr(torch, storage_dtype)
         self.mars, self.caution, self.mars_gamma = mars, caution, mars_gamma
         self.ecc, self.param_ecc = ecc, param_ecc
+        self.unfused = False  # True: the scale_by_* form of the transform even without update_clipping (MuonAdamW's vector route)
         self.rounding = rounding or HalfRounding()
         self.step_count = torch.zeros((), dtype=torch.int64)
         self.state = [dict() for _ in params]
@@ -461,7 +462,7 @@ class FirstOrderOracle:
                     u.copy_(c.to(u.dtype))
         m = [self._state_tensor(i, "exp_avg", grads[i].shape) for i in idx] if self.kind != "ademamix" else None
         v = [self._state_tensor(i, "exp_avg_sq", grads[i].shape) for i in idx]
-        if self.update_clipping is not None:
+        if self.update_clipping is not None or self.unfused:
             # un-fused chain (heavyball/chainable.py:2676-2701): scale_by_* leaves its result in the update buffer, which has the
             # gradient's dtype (copy_stochastic_list_: a stochastic round for bf16, heavyball/utils.py:1868, :2229, :2000, :2209,
             # :2327), the clip rewrites that buffer the same way (:3226-3232), update_param_ applies it (:2393-2406)
@@ -501,10 +502,11 @@ class FirstOrderOracle:
                                    apply=False)  # fmt: skip
             for u, n, t in zip(update, new, idx):
                 copy_stochastic(u, n, rounding, philox.STREAM_UPDATE, t)
-            fn = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip,
-                  "global_rmsnorm_clip": global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
-            for u, c, t in zip(update, fn(update), idx):
-                copy_stochastic(u, c, rounding, philox.STREAM_CLIP, t)
+            if self.update_clipping is not None:
+                fn = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip,
+                      "global_rmsnorm_clip": global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
+                for u, c, t in zip(update, fn(update), idx):
+                    copy_stochastic(u, c, rounding, philox.STREAM_CLIP, t)
             # the tail of the chain decays with the group's weight_decay whatever the transform did with it (NAdam: on top of its own)
             update_param_(p, update, lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)
             return

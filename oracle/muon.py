@@ -229,6 +229,7 @@ class MuonAdamWOracle:
         self.muon.KEY = "nesterov_ema_momentum_4" if nesterov else "exp_avg_exp_avg_4"
         self.adam = FirstOrderOracle("adam", list(params), eps=eps, rounding=self.rounding, **kw)
         self.adam.fn_name = "scale_by_adam"
+        self.adam.unfused = True  # heavyball/__init__.py:530-533: the route is scale_by_adam -> update_param_, never the fused form
         self.adam.mars_idx = 6  # behind the route's guards (trajectories written from the reference)
 
     @property

@@ -320,6 +320,8 @@ def test_muonadamw_matches_reference_trajectories_and_oracle():
             kwargs["betas"] = tuple(kwargs["betas"])
         n = len([k for k in d if k.startswith("init/p")])
         params = [torch.nn.Parameter(d[f"init/p{i}"].clone().to(DEV)) for i in range(n)]
+        for p in params:
+            p.grad_dtype = None  # bf16 gradients on fp32 parameters
         opt = heavyball_amd.MuonAdamW(params, **kwargs)
         opt.rounding = "half"
         orc = muon.MuonAdamWOracle([d[f"init/p{i}"].clone() for i in range(n)], rounding=HalfRounding(), **kwargs)
