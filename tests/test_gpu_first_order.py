@@ -121,20 +121,25 @@ def test_adopt_warmup_is_shared_by_the_tensors_of_a_step():
     assert not any(torch.equal(p.detach(), b) for p, b in zip(params, before))
 
 
-def test_bf16_params_plain():
-    """bf16 parameters without param_ecc: the parameter write is a stochastic round (heavyball/utils.py:2368-2369)."""
-    shapes = [(33, 9), (4100,)]
+@pytest.mark.parametrize("cls_name,kwargs", [("AdamW", dict(weight_decay=0.1)), ("AdamW", dict(storage_dtype="bfloat16", mars=True, caution=True)),
+                                             ("LaProp", dict(weight_decay=0.1, caution=True)), ("LaProp", dict(storage_dtype="bfloat16"))],
+                         ids=["adamw", "adamw_bf16_moments_mars_caution", "laprop_caution", "laprop_bf16_moments"])
+def test_bf16_params_plain(cls_name, kwargs):
+    """bf16 parameters without param_ecc: the parameter write is a stochastic round (heavyball/utils.py:2368-2369).  With
+    bf16 gradients over fp32 or bf16 moments: the mixed-precision set-ups that have kernels of their own."""
+    shapes = [(33, 9), (4100,), (8192 + 40,)]
+    cls, kind = CLS[cls_name]
     for rounding in ("half", "philox"):
         gen = torch.Generator().manual_seed(0)
         host = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
         params = [torch.nn.Parameter(h.clone().to(DEV)) for h in host]
-        opt = heavyball_amd.AdamW(params, weight_decay=0.1)
+        opt = cls(params, **kwargs)
         opt.rounding, opt.rng_seed = rounding, 5
         from oracle import first_order as fo
         from oracle.rounding import HalfRounding, PhiloxRounding
 
         r = HalfRounding() if rounding == "half" else PhiloxRounding(5, base=opt._buckets[0][0].slab.offsets_np.tolist())
-        orc = fo.FirstOrderOracle("adam", [h.clone() for h in host], weight_decay=0.1, rounding=r)
+        orc = fo.FirstOrderOracle(kind, [h.clone() for h in host], rounding=r, **kwargs)
         H.run_steps(opt, orc, params, shapes, 3, torch.bfloat16, 1e-2, DEV, tag="bf16 params " + rounding)
 
 
