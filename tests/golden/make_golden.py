@@ -331,7 +331,6 @@ def make_more_switches():
     for name, kw in [("soap_param_ecc_caution", dict(param_ecc="bf16+8", caution=True, precondition_frequency=3)),
                      ("soap_ecc", dict(ecc="bf16+8", precondition_frequency=3)),
                      ("soap_bf16_storage", dict(storage_dtype="bfloat16", precondition_frequency=3)),
-                     ("soap_split", dict(split=True, max_precond_dim=8, precondition_frequency=3)),
                      ("soap_precond_grad_accum", dict(precond_grad_accum=True, precondition_frequency=3))]:  # fmt: skip
         try:
             run_traj(name, heavyball.SOAP, kw, soap_shapes, torch.float32, 6)
