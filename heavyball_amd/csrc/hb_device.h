@@ -185,11 +185,16 @@ template <bool PRIM_BF16, bool CORR8>
 __device__ __forceinline__ int ecc_correction(float x, uint32_t h, uint32_t noise16) {
   const float e = x - prim_to_f32<PRIM_BF16>(h);
   const float en = ldexpf(e, -ecc_log_scale<PRIM_BF16>(h));
-  const float cl = __builtin_fminf(__builtin_fmaxf(en, -1.0f), 1.0f);
+  // A NaN (x is NaN, or x and its primary are the same infinity) goes through torch's clamp as NaN and becomes
+  // correction 0 in the conversion to the integer type; the hardware's min / max would turn it into -1 instead.
   if (CORR8) {
-    const int t = f2i_sat(cl * (127.0f * 65536.0f));
+    // clamp after the (saturating, NaN -> 0) conversion: the same integer for every finite en, since the conversion truncates
+    int t = f2i_sat(en * (127.0f * 65536.0f));
+    t = t < -127 * 65536 ? -127 * 65536 : (t > 127 * 65536 ? 127 * 65536 : t);
     return (t + (int)noise16) >> 16;
   } else {
+    float cl = __builtin_fminf(__builtin_fmaxf(en, -1.0f), 1.0f);
+    cl = en != en ? en : cl;
     const float scaled = cl * 32767.0f;
     return f2i_sat(__builtin_floorf(scaled + uniform16(noise16)));
   }

@@ -77,6 +77,29 @@ def test_encode_half_and_philox_match_oracle(mode):
         assert torch.equal(_decode(prim, corr, mode).view(torch.int32), e.decode().view(torch.int32))
 
 
+@pytest.mark.parametrize("mode", ["bf16+8", "bf16+16", "fp16+8", "fp16+16"])
+def test_encode_of_overflowing_and_non_finite_values_matches_oracle(mode):
+    """Values beyond the primary's range (1e5 in fp16), infinities and NaN: the primary overflows to infinity, and the
+    correction follows torch's arithmetic (clamp keeps a NaN, the conversion to the integer type makes it 0; a finite value
+    under an infinite primary gives -smax or +smax).  ADOPT's momentum, which divides by a root that can be 1e-8, gets
+    there on fp16 primaries."""
+    x = torch.tensor([float("inf"), float("-inf"), float("nan"), 1e5, -1e5, 65519.9, 65520.0, -65520.0, 3.4e38, -3.4e38, 3.3e38,
+                      1e-45, -1e-45, 0.0, -0.0, 1.0, 6e4] * 3)  # fmt: skip
+    for rng_mode in (_lib.RNG_HALF, _lib.RNG_PHILOX):
+        prim, corr = _encode(x, mode, rng_mode, seed=3, step=1, stream=2, base=64)
+        e = ecc.EccTensor.zeros(x.shape, mode)
+        if rng_mode == _lib.RNG_HALF:
+            u = torch.full(x.shape, 0.5)
+        else:
+            u = torch.from_numpy(philox.bits16(3, 1, 2, np.arange(64, 64 + x.numel(), dtype=np.uint64)).astype(np.float32)) / 65536.0
+        e.encode(x, u)
+        got_p, want_p = prim.cpu().float(), e.primary.float()
+        assert torch.equal(torch.isnan(got_p), torch.isnan(want_p))
+        ok = ~torch.isnan(want_p)
+        assert torch.equal(prim.cpu()[ok].view(torch.int16), e.primary[ok].view(torch.int16))
+        assert torch.equal(corr.cpu(), e.corr), (mode, rng_mode, corr.cpu().tolist(), e.corr.tolist())
+
+
 def test_exhaustive_bf16_patterns_roundtrip():
     """all 65,536 bf16 primaries x all 255 int8 corrections: GPU decode == oracle decode, bit for bit."""
     bits = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16)

@@ -184,6 +184,65 @@ def test_caution_count_on_updates_that_nearly_cancel(mars, rounding):
         H.compare(opt, orc, params, f"nearly cancelling step {k}")
 
 
+def _random_case(seed):
+    """One draw from the switches the five fused optimizers share, on ragged shapes around the chunk and work-unit sizes."""
+    import random
+
+    rnd = random.Random(seed)
+    cls_name = rnd.choice(["AdamW", "LaProp", "ADOPT", "AdEMAMix", "NAdam"])
+    kwargs = dict(mars=rnd.random() < 0.4, caution=rnd.random() < 0.4)
+    if rnd.random() < 0.5:
+        kwargs["weight_decay"] = rnd.choice([0.01, 0.1])
+        kwargs["cautious_weight_decay"] = rnd.random() < 0.3
+    if rnd.random() < 0.3:
+        kwargs["warmup_steps"] = rnd.choice([1, 3])
+    if rnd.random() < 0.2 and cls_name != "AdEMAMix":
+        kwargs["palm"] = True
+    storage = rnd.choice(["f32", "bf16", "bf16+8", "bf16+8", "bf16+16", "fp16+8", "fp16+16"])
+    if "+" in storage:
+        kwargs["ecc"] = storage
+    elif storage == "bf16":
+        kwargs["storage_dtype"] = "bfloat16"
+    gdt = rnd.choice([torch.float32, torch.bfloat16, torch.bfloat16, torch.float16])
+    bf16_params = False
+    pe = rnd.choice([None, None, "bf16+8", "fp16+16", "bf16+16"])
+    if pe is not None:
+        kwargs["param_ecc"] = pe
+    elif gdt == torch.bfloat16 and rnd.random() < 0.4:
+        bf16_params = True
+    if cls_name == "NAdam" and rnd.random() < 0.5:
+        kwargs["decoupled_weight_decay"] = True
+    sizes = [1, 7, 8, 9, 255, 256, 257, 1023, 1024, 2047, 2048, 2049, 4095, 4096, 4097, 6143, 8191, 8192, 8193, 12345]
+    shapes = [(rnd.choice(sizes),) for _ in range(rnd.randint(2, 5))] + [(rnd.randint(1, 70), rnd.randint(1, 90))]
+    rnd.shuffle(shapes)
+    none_for = {2: [rnd.randrange(len(shapes))]} if rnd.random() < 0.3 else None
+    return cls_name, kwargs, gdt, bf16_params, shapes, none_for, rnd.choice(["half", "philox"])
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_configurations_match_oracle(seed):
+    """Seeded draws over optimizer, switches, storage formats, gradient and parameter dtypes and ragged sizes (one element up
+    to three chunks, around every multiple of the work unit), three steps each, bit for bit against the oracle: the
+    combinations nobody listed by hand, most of them on the kernel that switches on run-time format codes."""
+    from oracle import first_order as fo
+    from oracle.rounding import HalfRounding, PhiloxRounding
+
+    cls_name, kwargs, gdt, bf16_params, shapes, none_for, rounding = _random_case(seed)
+    print("case", seed, cls_name, kwargs, gdt, "bf16 params" if bf16_params else "", shapes, none_for, rounding, flush=True)
+    cls, kind = CLS[cls_name]
+    if not bf16_params:
+        host, params, opt, orc = H.build_pair(cls, kind, shapes, kwargs, DEV, rounding=rounding)
+    else:
+        gen = torch.Generator().manual_seed(0)
+        host = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
+        params = [torch.nn.Parameter(h.clone().to(DEV)) for h in host]
+        opt = cls(params, **kwargs)
+        opt.rounding, opt.rng_seed = rounding, 77
+        r = HalfRounding() if rounding == "half" else PhiloxRounding(77, base=opt._buckets[0][0].slab.offsets_np.tolist())
+        orc = fo.FirstOrderOracle(kind, [h.clone() for h in host], rounding=r, **kwargs)
+    H.run_steps(opt, orc, params, shapes, 3, gdt, 1e-2 if gdt == torch.float32 else 1e-3, DEV, none_for=none_for, tag=f"draw {seed}")
+
+
 def test_c1_full_size():
     """Benchmark configuration 1 at its full size: 4 fp32 tensors, 9,438,208 elements, 10 steps, bit-exact against the oracle."""
     shapes = [(1024, 1024), (1024,), (4096, 1024), (1024, 4096)]
