@@ -176,9 +176,10 @@ __device__ __forceinline__ int f2i_sat(float x) {
 
 // correction of x against its primary h: floor(clamp((x - primary) * 2^-ls, -1, 1) * smax + u), u = noise16 / 65536.
 //
-// int8: e = x - primary has at most 16 significant bits, so scaled = clamp(..) * 127 is exact in fp32 with at most 15
-// fractional bits, scaled + u is exact as well, and floor(scaled + k / 65536) == (scaled * 65536 + k) >> 16 in integers:
-// one multiply, one convert, one add and one shift replace convert + multiply + add + floor + convert.
+// int8 on a bf16 primary: e = x - primary has at most 16 significant bits (also when x or the primary is denormal), so
+// scaled = clamp(..) * 127 is exact in fp32 with at most 15 fractional bits, scaled + u is exact as well, and
+// floor(scaled + k / 65536) == (scaled * 65536 + k) >> 16 in integers: one multiply, one convert, one add and one shift
+// replace convert + multiply + add + floor + convert.
 // int16: scaled has up to 31 significant bits before the add, so the reference's fp32 rounding of (scaled + u) matters
 // and the float formulation is kept.
 template <bool PRIM_BF16, bool CORR8>
@@ -187,15 +188,18 @@ __device__ __forceinline__ int ecc_correction(float x, uint32_t h, uint32_t nois
   const float en = ldexpf(e, -ecc_log_scale<PRIM_BF16>(h));
   // A NaN (x is NaN, or x and its primary are the same infinity) goes through torch's clamp as NaN and becomes
   // correction 0 in the conversion to the integer type; the hardware's min / max would turn it into -1 instead.
-  if (CORR8) {
+  if (CORR8 && PRIM_BF16) {
     // clamp after the (saturating, NaN -> 0) conversion: the same integer for every finite en, since the conversion truncates
     int t = f2i_sat(en * (127.0f * 65536.0f));
     t = t < -127 * 65536 ? -127 * 65536 : (t > 127 * 65536 ? 127 * 65536 : t);
     return (t + (int)noise16) >> 16;
   } else {
+    // fp16 primaries: below the smallest normal fp16 value (6e-5: second moments of small gradients live there) the residual
+    // keeps up to 24 significant bits, scaled is rounded, and only the reference's own fp32 sequence reproduces it
+    constexpr float smax = CORR8 ? 127.0f : 32767.0f;
     float cl = __builtin_fminf(__builtin_fmaxf(en, -1.0f), 1.0f);
     cl = en != en ? en : cl;
-    const float scaled = cl * 32767.0f;
+    const float scaled = cl * smax;
     return f2i_sat(__builtin_floorf(scaled + uniform16(noise16)));
   }
 }

@@ -60,7 +60,10 @@ def test_decode_matches_reference_vectors(mode):
 def test_encode_half_and_philox_match_oracle(mode):
     d = torch.load(os.path.join(GOLDEN, "ecc.pt"), weights_only=True)
     gen = torch.Generator().manual_seed(7)
-    x = torch.cat([d["x"], torch.randn(100_003, generator=gen) * torch.exp(torch.randn(100_003, generator=gen) * 4)])
+    x = torch.cat([d["x"], torch.randn(100_003, generator=gen) * torch.exp(torch.randn(100_003, generator=gen) * 4),
+                   # second moments of small gradients: below the smallest normal fp16 value, where the residual against an fp16
+                   # primary keeps up to 24 significant bits and the correction depends on every rounding of the reference's sequence
+                   torch.randn(400_000, generator=gen).square() * 1e-6, torch.randn(100_000, generator=gen) * 3e-8])
     if mode.startswith("fp16"):
         x = x.clamp(-6e4, 6e4)
     for rng_mode, base in ((_lib.RNG_HALF, 0), (_lib.RNG_PHILOX, 8 * 12345 + 3)):
