@@ -335,6 +335,22 @@ def palm_betas(betas, step: Tensor, beta2_scale: float):
     return (betas[0], beta2, *betas[2:])
 
 
+def narrow_params(params, param_ecc, rounding):
+    """heavyball/chainable.py:2421-2444: param_ecc narrows the live parameter at construction (a parameter that already is an
+    EccTensor, or param_ecc None: unchanged)."""
+    out = []
+    for i, p in enumerate(params):
+        if param_ecc is None or isinstance(p, EccTensor):
+            out.append(p)
+            continue
+        pd, cd = MODES[param_ecc]
+        e = EccTensor(p.to(pd), torch.zeros(p.shape, dtype=cd))
+        if p.dtype != pd:
+            e.compute_correction(p.float(), rounding.at_step(0).uniform(philox.STREAM_INIT_PARAM, i, p.shape))
+        out.append(e)
+    return out
+
+
 class FirstOrderOracle:
     """AdamW or LaProp over a list of tensors, with the reference's state layout.
 
@@ -398,19 +414,10 @@ class FirstOrderOracle:
         self.rounding = rounding or HalfRounding()
         self.step_count = torch.zeros((), dtype=torch.int64)
         self.state = [dict() for _ in params]
-        self.params = []
-        # heavyball/chainable.py:2421-2444: param_ecc narrows the live parameter at construction
-        for i, p in enumerate(params):
-            if param_ecc is None:
-                self.params.append(p)
-                continue
-            pd, cd = MODES[param_ecc]
-            e = EccTensor(p.to(pd), torch.zeros(p.shape, dtype=cd))
-            if p.dtype != pd:
-                r = self.rounding.at_step(0)
-                e.compute_correction(p.float(), r.uniform(philox.STREAM_INIT_PARAM, i, p.shape))
-            self.params.append(e)
-            self.state[i]["param::ecc"] = e.corr
+        self.params = narrow_params(params, param_ecc, self.rounding)
+        for i, e in enumerate(self.params):
+            if isinstance(e, EccTensor):
+                self.state[i]["param::ecc"] = e.corr
 
     def key(self, name):
         idx = {"mars_old_grad": self.mars_idx, "mu_product": 1}.get(name, 0)

@@ -118,8 +118,12 @@ class MuonOracle:
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), weight_decay=0.0, warmup_steps=0, caution=False,
                  cautious_weight_decay=False, rounding=None, mode="newtonschulz", nesterov=True, heavyball_momentum=False,
-                 gradient_clipping=None, update_clipping=None, ecc=None, storage_dtype="float32", mars=False, mars_gamma=0.0025):  # fmt: skip
-        self.params = params
+                 gradient_clipping=None, update_clipping=None, ecc=None, storage_dtype="float32", mars=False, mars_gamma=0.0025,
+                 param_ecc=None):  # fmt: skip
+        from .first_order import narrow_params
+
+        self.rounding = rounding or HalfRounding()
+        self.params = narrow_params(params, param_ecc, self.rounding)
         self.mars, self.mars_gamma = mars, mars_gamma
         self.ecc, self.storage_dtype = ecc, getattr(torch, storage_dtype)
         self.gradient_clipping, self.update_clipping = gradient_clipping, update_clipping
@@ -130,9 +134,11 @@ class MuonOracle:
             self.KEY = "exp_avg_exp_avg_2"
         self.lr, self.betas, self.weight_decay, self.warmup_steps = lr, betas, weight_decay, warmup_steps
         self.caution, self.cautious_weight_decay = caution, cautious_weight_decay
-        self.rounding = rounding or HalfRounding()
         self.mode = mode
         self.state = [dict() for _ in params]
+        for i, e in enumerate(self.params):
+            if isinstance(e, EccTensor):
+                self.state[i]["param::ecc"] = e.corr
         self.step_count = torch.zeros((), dtype=torch.int64)
 
     KEY = "nesterov_ema_momentum_2"
@@ -148,7 +154,7 @@ class MuonOracle:
         st = self.state[i]
         if key not in st:
             if self.ecc is None:
-                st[key] = torch.zeros_like(self.params[i], dtype=self.storage_dtype)
+                st[key] = torch.zeros(tuple(self.params[i].shape), dtype=self.storage_dtype)
             else:
                 e = EccTensor.zeros(self.params[i].shape, self.ecc)
                 st[key], st[key + "::ecc"] = e.primary, e.corr
@@ -213,8 +219,8 @@ class MuonAdamWOracle:
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), eps=1e-8, weight_decay=0.0, warmup_steps=0, caution=False,
                  cautious_weight_decay=False, rounding=None, mars=False, mars_gamma=0.0025, ecc=None, storage_dtype="float32",
-                 nesterov=True, gradient_clipping=None, update_clipping=None):  # fmt: skip
-        from .first_order import FirstOrderOracle
+                 nesterov=True, gradient_clipping=None, update_clipping=None, param_ecc=None):  # fmt: skip
+        from .first_order import FirstOrderOracle, narrow_params
 
         for kind in (gradient_clipping, update_clipping):
             assert kind in (None, "l2_clip_", "rmsnorm_clip_"), "a norm over the whole group would span both routes"
@@ -222,6 +228,7 @@ class MuonAdamWOracle:
         self.mat_idx = [i for i, p in enumerate(params) if p.dim() >= 2]
         self.vec_idx = [i for i, p in enumerate(params) if p.dim() < 2]
         self.rounding = rounding or HalfRounding()
+        params = self.params = narrow_params(params, param_ecc, self.rounding)  # both routes work on the narrowed parameters
         kw = dict(lr=lr, betas=betas, weight_decay=weight_decay, warmup_steps=warmup_steps, caution=caution,
                   cautious_weight_decay=cautious_weight_decay, mars=mars, mars_gamma=mars_gamma, ecc=ecc, storage_dtype=storage_dtype,
                   gradient_clipping=gradient_clipping, update_clipping=update_clipping)  # fmt: skip

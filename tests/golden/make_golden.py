@@ -316,6 +316,8 @@ def make_more_switches():
              4, grad_scale=1.0)  # fmt: skip
     run_traj("muonadamw_ecc_updclip", heavyball.MuonAdamW, dict(ecc="bf16+8", update_clipping="rmsnorm_clip_"), shapes, torch.float32, 4)
     run_traj("muonadamw_plain_ema_bf16_storage", heavyball.MuonAdamW, dict(nesterov=False, storage_dtype="bfloat16"), shapes, torch.float32, 4)
+    run_traj("muon_param_ecc_caution", heavyball.Muon, dict(param_ecc="bf16+8", caution=True, weight_decay=0.01), shapes, torch.float32, 4)
+    run_traj("muonadamw_param_ecc16_mars", heavyball.MuonAdamW, dict(param_ecc="bf16+16", mars=True), shapes, torch.float32, 4)
     # bf16 gradients: the un-fused scale_by_adam of the vector route writes its result into a bf16 update buffer
     run_traj("muonadamw_bf16grad_ecc_caution", heavyball.MuonAdamW, dict(ecc="bf16+8", caution=True, weight_decay=0.01), shapes, torch.bfloat16, 4)
     soap_shapes = [(8, 16), (16,), (12, 6)]

@@ -250,6 +250,98 @@ def test_muon_optimizer_matches_oracle(variant, rounding):
         assert opt.param_groups[0]["step"] is None
 
 
+def _random_muon_case(seed):
+    import random
+
+    rnd = random.Random(1000 + seed)
+    kwargs = dict(lr=0.02, nesterov=rnd.random() < 0.6, heavyball_momentum=rnd.random() < 0.3, mars=rnd.random() < 0.4,
+                  caution=rnd.random() < 0.4, betas=(rnd.choice([0.9, 0.95]), 0.99))  # fmt: skip
+    if rnd.random() < 0.5:
+        kwargs["weight_decay"] = rnd.choice([0.01, 0.1])
+        kwargs["cautious_weight_decay"] = rnd.random() < 0.3
+    storage = rnd.choice(["f32", "f32", "bf16", "bf16+8", "bf16+16", "fp16+8", "fp16+16"])
+    if "+" in storage:
+        kwargs["ecc"] = storage
+    elif storage == "bf16":
+        kwargs["storage_dtype"] = "bfloat16"
+    if rnd.random() < 0.3:
+        kwargs["param_ecc"] = rnd.choice(["bf16+8", "bf16+16"])
+    gdt = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+    dims = [1, 2, 7, 8, 33, 64, 127, 128, 129, 200, 256, 300]
+    shapes = [(rnd.choice(dims), rnd.choice(dims)) for _ in range(rnd.randint(2, 4))] + [(rnd.choice([1, 9, 64, 4097]),)]
+    if rnd.random() < 0.4:
+        shapes.append((rnd.randint(2, 6), rnd.randint(2, 6), rnd.choice([8, 24, 31])))
+    rnd.shuffle(shapes)
+    return kwargs, gdt, shapes, rnd.choice(["half", "philox"])
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_muon_configurations_match_oracle(seed):
+    """Seeded draws over Muon's momentum forms, MARS, caution, decay, storage of the momentum and of the parameter, gradient
+    dtype and shapes (vectors, thin and tiny matrices, stacks): momentum, MARS' old gradient and their corrections bit for
+    bit, vectors bit for bit, matrices to the Newton-Schulz tolerance on the step taken."""
+    from oracle.ecc import EccTensor
+    from tests import helpers as H
+
+    kwargs, gdt, shapes, rounding = _random_muon_case(seed)
+    print("case", seed, kwargs, gdt, shapes, rounding, flush=True)
+    host, params, opt, orc = _muon_pair(shapes, kwargs, rounding)
+    if kwargs.get("param_ecc"):
+        for b in opt._buckets[0]:
+            for i, p in enumerate(b.params):
+                j = [id(q) for q in params].index(id(p))
+                opt._encode_param(b, i, host[j].to(DEV).contiguous(), opt.param_groups[0])
+
+    def value(t, corr):
+        t = t.detach().cpu()
+        return EccTensor(t, corr.detach().cpu()).decode() if corr is not None else t.float()
+
+    for k in range(1, 4):
+        grads = H.make_grads(shapes, k, gdt, 1e-2)
+        prev = [value(p.data, opt.state[p][0].get("param::ecc") if p in opt.state and 0 in opt.state[p] else None) for p in params]
+        prev_o = [q.decode() if isinstance(q, EccTensor) else q.clone() for q in orc.params]
+        for p, g in zip(params, grads):
+            p.grad = g.to(DEV)
+        opt.step()
+        orc.step([g.clone() for g in grads])
+        torch.cuda.synchronize()
+        for i, p in enumerate(params):
+            st = opt.state[p][0]
+            for key, val in orc.state[i].items():
+                if isinstance(val, torch.Tensor) and key not in ("step", "param::ecc"):
+                    H.assert_bit_equal(st[key], val, f"step {k} tensor {i} {key}")
+            q = orc.params[i]
+            if p.dim() < 2:
+                H.assert_bit_equal(p.data, q.primary if isinstance(q, EccTensor) else q, f"step {k} vector {i}")
+                if isinstance(q, EccTensor):
+                    H.assert_bit_equal(st["param::ecc"], q.corr, f"step {k} vector {i} correction")
+            else:
+                got = value(p.data, st.get("param::ecc")) - prev[i]
+                want = (q.decode() if isinstance(q, EccTensor) else q) - prev_o[i]
+                # a parameter kept as an ECC pair moves in units of 2^-8/127 of a bf16 ulp: allow that resolution on top
+                slack = 4 * (2.0**-8 / 127) * prev[i].abs().max().item() * prev[i].numel() ** 0.5 if kwargs.get("param_ecc") else 0.0
+                assert (got - want).norm().item() <= NS_TOL * want.norm().item() + slack, (k, i, rel_fro(got, want))
+
+
+def _matrix_step_close(d, k, i, p, st):
+    """The step a matrix took against the fixture's, to the Newton-Schulz tolerance; ECC parameters are decoded first (the fixture
+    holds no correction for the narrowed initial parameter, so their first step has no reference point)."""
+    from oracle.ecc import EccTensor
+
+    def full(t, key):
+        return EccTensor(t, d[key]).decode() if key in d else t.float()
+
+    if f"step{k}/state{i}/param::ecc" in d:
+        if k == 1:
+            return
+        got = EccTensor(p.detach().cpu(), st["param::ecc"].cpu()).decode()
+    else:
+        got = p.detach().cpu()
+    prev = full(d[f"step{k - 1}/p{i}"], f"step{k - 1}/state{i}/param::ecc") if k > 1 else d[f"init/p{i}"]
+    want = full(d[f"step{k}/p{i}"], f"step{k}/state{i}/param::ecc")
+    assert rel_fro(got - prev, want - prev) < NS_TOL, (k, i, rel_fro(got - prev, want - prev))
+
+
 def test_muon_matches_reference_trajectories():
     import glob
     import json
@@ -266,7 +358,11 @@ def test_muon_matches_reference_trajectories():
         params = [torch.nn.Parameter(d[f"init/p{i}"].clone().to(DEV)) for i in range(n)]
         for p in params:
             p.grad_dtype = None  # bf16 gradients on fp32 parameters
-        opt = heavyball_amd.Muon(params, **kwargs)
+        heavyball_amd.HBOptimizer.rounding = "half"  # param_ecc encodes the parameters at construction
+        try:
+            opt = heavyball_amd.Muon(params, **kwargs)
+        finally:
+            heavyball_amd.HBOptimizer.rounding = "philox"
         opt.rounding = "half"
         for k in range(1, d["meta/steps"] + 1):
             for i, p in enumerate(params):
@@ -279,10 +375,10 @@ def test_muon_matches_reference_trajectories():
                 prefix = f"step{k}/state{i}/"
                 want_state = {kk[len(prefix):]: d[kk] for kk in d if kk.startswith(prefix) and not kk.endswith("/step")}
                 assert set(want_state) == {kk for kk in opt.state[p][0] if kk not in ("step", "is_initialized")}
-                for kk, vv in want_state.items():  # ECC corrections and MARS' old gradient have to match too
-                    if kk != opt.KEY:
-                        assert torch.equal(opt.state[p][0][kk].cpu(), vv), (k, i, kk)
                 want, prev = d[f"step{k}/p{i}"], (d[f"step{k - 1}/p{i}"] if k > 1 else d[f"init/p{i}"])
+                for kk, vv in want_state.items():  # ECC corrections and MARS' old gradient have to match too
+                    if kk != opt.KEY and not (kk == "param::ecc" and want.dim() >= 2):
+                        assert torch.equal(opt.state[p][0][kk].cpu(), vv), (k, i, kk)
                 if "clip" in path:  # the clip norm is summed in another order: 2e-6 of the tensor's scale instead of equality
                     assert ((got_mom - mom).abs() <= 2e-6 * (mom.abs() + mom.abs().max())).all()
                     if want.dim() < 2:
@@ -293,7 +389,7 @@ def test_muon_matches_reference_trajectories():
                 if want.dim() < 2:
                     assert torch.equal(p.detach().cpu(), want)
                 else:
-                    assert rel_fro(p.detach().cpu() - prev, want - prev) < NS_TOL
+                    _matrix_step_close(d, k, i, p, opt.state[p][0])
         sd = opt.state_dict()
         assert set(sd["state"][0][0].keys()) >= {opt.KEY, "is_initialized", "step"}
         want_init = set(d["final/is_initialized0"].tolist()) if "final/is_initialized0" in d else {0, 1, 2}
@@ -322,7 +418,11 @@ def test_muonadamw_matches_reference_trajectories_and_oracle():
         params = [torch.nn.Parameter(d[f"init/p{i}"].clone().to(DEV)) for i in range(n)]
         for p in params:
             p.grad_dtype = None  # bf16 gradients on fp32 parameters
-        opt = heavyball_amd.MuonAdamW(params, **kwargs)
+        heavyball_amd.HBOptimizer.rounding = "half"  # param_ecc encodes the parameters at construction
+        try:
+            opt = heavyball_amd.MuonAdamW(params, **kwargs)
+        finally:
+            heavyball_amd.HBOptimizer.rounding = "philox"
         opt.rounding = "half"
         orc = muon.MuonAdamWOracle([d[f"init/p{i}"].clone() for i in range(n)], rounding=HalfRounding(), **kwargs)
         for k in range(1, d["meta/steps"] + 1):
@@ -343,15 +443,18 @@ def test_muonadamw_matches_reference_trajectories_and_oracle():
                     check = H.assert_close_in_scale if "clip" in path else H.assert_close_to_reference
                     check({"param": p.data, **st}, {"param": want, **want_state}, f"step {k} vector {i}")
                     if "clip" not in path:  # a clip norm is summed in another order than the oracle's
-                        H.assert_bit_equal(p.data, orc.params[i], f"step {k} vector {i} vs oracle")
+                        q = orc.params[i]
+                        H.assert_bit_equal(p.data, q.primary if hasattr(q, "primary") else q, f"step {k} vector {i} vs oracle")
                     assert st["is_initialized"] == (set(d[fk].tolist()) if fk in d else {0})
                 else:
                     for kk, vv in want_state.items():
+                        if kk == "param::ecc":
+                            continue
                         if "clip" in path and "updclip" not in path:  # gradient clipping ahead of the momentum
                             assert ((st[kk].cpu().float() - vv.float()).abs() <= 2e-6 * (vv.float().abs() + vv.float().abs().max())).all(), (k, i, kk)
                         else:
                             assert torch.equal(st[kk].cpu(), vv), (k, i, kk)
-                    assert rel_fro(p.detach().cpu() - prev, want - prev) < NS_TOL
+                    _matrix_step_close(d, k, i, p, st)
                     assert st["is_initialized"] == (set(d[fk].tolist()) if fk in d else {2, 3, 4})
 
 
