@@ -450,6 +450,36 @@ def test_soap_narrow_storage_matches_oracle(kwargs, rounding):
                 assert torch.equal(opt.state[p][0][km], opt2.state[p2][0][km])
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_soap_configurations_match_oracle(seed):
+    """Seeded draws over SOAP's switches (MARS, caution, decay, max_precond_dim down to sizes that drop a side, precondition_1d,
+    the four clip kinds on the gradient and on the update) and shapes (matrices of aspect ratio at most 2, so that both
+    factors have full rank by the first refresh and the refreshed basis is determined by the data; vectors; a stack that
+    is merged), seven steps with two refreshes, the step to 5e-3 against the oracle."""
+    import random
+
+    rnd = random.Random(5000 + seed)
+    kwargs = dict(precondition_frequency=rnd.choice([3, 4]), mars=rnd.random() < 0.3, caution=rnd.random() < 0.3,
+                  weight_decay=rnd.choice([0.0, 0.01, 0.1]), max_precond_dim=rnd.choice([2048, 2048, 64, 24, 10]),
+                  precondition_1d=rnd.random() < 0.3)  # fmt: skip
+    if rnd.random() < 0.25 and not kwargs["mars"]:
+        kwargs["gradient_clipping"] = rnd.choice(["l2_clip_", "rmsnorm_clip_", "global_l2norm_clip", "global_rmsnorm_clip"])
+    if rnd.random() < 0.25:
+        kwargs["update_clipping"] = rnd.choice(["l2_clip_", "rmsnorm_clip_", "global_l2norm_clip", "global_rmsnorm_clip"])
+    shapes = []
+    for _ in range(rnd.randint(1, 3)):
+        a = rnd.choice([2, 5, 8, 16, 24, 33, 40, 64])
+        shapes.append((a, rnd.randint(max(1, (a + 1) // 2), 2 * a)))
+    shapes.append((rnd.choice([1, 2, 3]) if kwargs["precondition_1d"] else rnd.choice([1, 3, 17, 70]),))
+    if rnd.random() < 0.5:
+        shapes.append((rnd.choice([4, 6]), 2, rnd.choice([2, 3])))
+    if rnd.random() < 0.2:
+        shapes.append(())
+    rnd.shuffle(shapes)
+    print("case", seed, kwargs, shapes, flush=True)
+    _run_soap_vs_oracle(shapes, kwargs, 7, 5e-3)
+
+
 def test_soap_and_muon_step_over_empty_scalar_and_degenerate_tensors():
     """Zero-sized tensors are skipped, 0-d and 1-element tensors and matrices with a dimension of 1 (which get no factor)
     step and stay finite; no launch is attempted with an empty grid."""
