@@ -316,6 +316,56 @@ def test_state_dict_roundtrip_continues_identically():
         assert opt2.state[b][0]["update_by_adam_exp_avg_0::ecc"].dtype == torch.int8
 
 
+@pytest.mark.parametrize("rounding", ["half", "philox"])
+def test_param_groups_step_independently(rounding):
+    """Two parameter groups with their own lr, betas and weight decay, one of them without gradients at step 2, and a third
+    group added after construction: every group keeps its own step counter (heavyball/chainable.py:2531-2570), so each
+    behaves like an optimizer of its own over the steps in which it had gradients.  Bit for bit against one oracle per group."""
+    from oracle import first_order as fo
+    from oracle.rounding import HalfRounding, PhiloxRounding
+
+    shapes = [[(130, 33), (4100,)], [(8193,)], [(77,), (5, 9)]]
+    common = dict(ecc="bf16+8", caution=True)
+    per_group = [dict(lr=1e-3, weight_decay=0.1), dict(lr=3e-3, betas=(0.8, 0.95)), dict(lr=2e-3, mars=True, weight_decay=0.01)]
+    gen = torch.Generator().manual_seed(4)
+    host = [[torch.randn(s, generator=gen) * 0.02 for s in grp] for grp in shapes]
+    params = [[torch.nn.Parameter(h.clone().to(DEV)) for h in grp] for grp in host]
+    for grp in params:
+        for p in grp:
+            p.grad_dtype = None
+    opt = heavyball_amd.AdamW([dict(params=params[0], **per_group[0]), dict(params=params[1], **per_group[1])], **common)
+    opt.rounding, opt.rng_seed = rounding, 9
+    opt.add_param_group(dict(params=params[2], **per_group[2]))
+    assert len(opt.param_groups) == 3 and opt.param_groups[2]["ecc"] == "bf16+8" and opt.param_groups[2]["mars"] is True
+    oracles = []
+    for gi in range(3):
+        base = opt._buckets[gi][0].slab.offsets_np.tolist() if gi in opt._buckets else None
+        r = HalfRounding() if rounding == "half" else None
+        oracles.append([fo, host[gi], {**common, **per_group[gi]}, r, base])
+    built = {}
+    for k in range(1, 5):
+        for gi in range(3):
+            has_grads = not (gi == 1 and k == 2)
+            grads = H.make_grads(shapes[gi], 10 * gi + k, torch.bfloat16, 1e-3) if has_grads else [None] * len(shapes[gi])
+            for p, g in zip(params[gi], grads):
+                p.grad = None if g is None else g.to(DEV)
+            oracles[gi].append(grads)
+        opt.step()
+        torch.cuda.synchronize()
+        for gi in range(3):
+            if gi not in built:  # the slab offsets (the noise generator's index base) exist once the group has stepped
+                _, h, kw, r, _ = oracles[gi][:5]
+                if r is None:
+                    r = PhiloxRounding(9, base=opt._buckets[gi][0].slab.offsets_np.tolist())
+                built[gi] = fo.FirstOrderOracle("adam", [t.clone() for t in h], rounding=r, **kw)
+            grads = oracles[gi][-1]
+            if any(g is not None for g in grads):
+                built[gi].step([None if g is None else g.clone() for g in grads])
+            H.compare(opt, built[gi], params[gi], f"group {gi} step {k}")
+    steps = [int(opt.state[grp[0]][0]["step"]) for grp in params]
+    assert steps == [4, 3, 4], steps
+
+
 def test_error_paths():
     L = _lib.lib()
     d = _lib.HbStepDesc()
