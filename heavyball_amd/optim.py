@@ -227,6 +227,15 @@ class HBOptimizer(torch.optim.Optimizer):
             self._adopt_group(gi, group)
 
     # -- construction -------------------------------------------------------------------------------------------
+    def _betas(self, group, step):
+        beta1 = group["betas"][0] if group.get("beta") is None else group["beta"]
+        if self._use_palm:  # heavyball/chainable.py:1921-1925
+            beta2 = 1 - group["step"] ** -group["beta2_scale"]
+            group["betas"] = (beta1, beta2, *group["betas"][2:])
+        else:
+            beta2 = group["betas"][1]
+        return f32(beta1), f32(beta2)
+
     @staticmethod
     def _pick(a, b):
         return b if a is use_default else a
@@ -670,15 +679,6 @@ class FirstOrder(HBOptimizer):
                     st.setdefault(k + "::ecc", b.slab.view(k + "::ecc", i))
             st.setdefault("is_initialized", set()).update(init_ids)
         ready.update(idx)
-
-    def _betas(self, group, step):
-        beta1 = group["betas"][0] if group.get("beta") is None else group["beta"]
-        if self._use_palm:  # heavyball/chainable.py:1921-1925
-            beta2 = 1 - group["step"] ** -group["beta2_scale"]
-            group["betas"] = (beta1, beta2, *group["betas"][2:])
-        else:
-            beta2 = group["betas"][1]
-        return f32(beta1), f32(beta2)
 
     def _step_scalars(self, group, step) -> dict:
         """The fp32 scalars of the step as the reference's 0-d tensors hold them (descriptor field -> python float)."""

@@ -129,16 +129,15 @@ class SOAP(HBOptimizer):
                  promote: bool = use_default, ecc: Optional[str] = None, param_ecc: Optional[str] = None, orig_shapes=None, **kwargs):  # fmt: skip
         params, defaults = build_defaults(locals())
         if defaults.pop("use_precond_schedule") not in (use_default, False):
-            raise NotImplementedError("SOAP: use_precond_schedule")
+            # the reference cannot run it either: heavyball/utils.py:3497 hands the schedule a python int and :2411 calls .clamp on it
+            raise NotImplementedError("SOAP: use_precond_schedule (the reference's own schedule fails on its first call)")
         del defaults["precond_scheduler"]
         self.precond_schedule = 1 / defaults.pop("precondition_frequency")  # heavyball/__init__.py:842-858
         # precond_grad_accum is read by PSGD's guard only (heavyball/chainable.py:304-345): SOAP's chain ignores it, and so does this
-        if split or not merge_dims:
-            raise NotImplementedError("SOAP on the HIP kernels: split and merge_dims=False are not built")
+        if split:
+            raise NotImplementedError("SOAP on the HIP kernels: split (one state per block of a parameter) is not built")
         if mars and (ecc or storage_dtype != "float32"):
             raise NotImplementedError("SOAP on the HIP kernels: mars together with ecc or non-fp32 storage")
-        if palm not in (use_default, False):
-            raise NotImplementedError("SOAP on the HIP kernels: palm (the beta2 schedule of heavyball/chainable.py:1921-1925) is not built")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
         if mars and self.gradient_clipping is not None:
             raise NotImplementedError("SOAP on the HIP kernels: mars together with gradient_clipping")
@@ -150,7 +149,7 @@ class SOAP(HBOptimizer):
         L = _lib.lib()
         step = group["step"]
         lr = f32(group["lr"])
-        beta1, beta2 = f32(group["betas"][0]), f32(group["betas"][1])
+        beta1, beta2 = self._betas(group, step)
         adam_step = step - 1  # heavyball/chainable.py:1270
         max_dim = group["max_precond_dim"]
         decay = group["weight_decay"]
@@ -208,7 +207,8 @@ class SOAP(HBOptimizer):
             with torch.cuda.device(b.device):
                 for (i, p, g), g32 in zip(items, raw[key]):
                     keep.append(g32)
-                    shape = merged_shape(p.shape, max_dim) if p.dim() > 0 else []
+                    # heavyball/utils.py:3726-3742: without merge_dims the parameter is taken as it is
+                    shape = (merged_shape(p.shape, max_dim) if group.get("merge_dims", True) else list(p.shape)) if p.dim() > 0 else []
                     G0 = g32.reshape(shape) if shape else g32.reshape(1)  # the gradient
                     G = b.slab.view("_clip", i).reshape(G0.shape) if self.gradient_clipping is not None else G0  # the update
                     st = self._state0(p)

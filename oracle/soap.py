@@ -153,12 +153,13 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
 
 
 class SOAPOracle:
-    """heavyball.SOAP (heavyball/__init__.py:861-909) with merge_dims=True, split=False."""
+    """heavyball.SOAP (heavyball/__init__.py:861-909) with split=False."""
 
     def __init__(self, params, lr=3e-3, betas=(0.9, 0.95), shampoo_beta=0.95, eps=1e-8, weight_decay=0.01, precondition_frequency=2,
                  max_precond_dim=2048, precondition_1d=False, warmup_steps=0, gradient_clipping=None,
                  update_clipping=None, mars=False, mars_gamma=0.0025, ecc=None, storage_dtype="float32", param_ecc=None,
-                 caution=False, cautious_weight_decay=False, precond_grad_accum=False, rounding=None):  # fmt: skip
+                 caution=False, cautious_weight_decay=False, precond_grad_accum=False, palm=False, beta2_scale=0.8, merge_dims=True,
+                 rounding=None):  # fmt: skip
         from . import philox
         from .ecc import MODES, EccTensor
         from .rounding import HalfRounding
@@ -169,6 +170,7 @@ class SOAPOracle:
         self.caution, self.cautious_weight_decay = caution, cautious_weight_decay
         self.param_ecc = param_ecc
         self.mars, self.mars_gamma = mars, mars_gamma
+        self.palm, self.beta2_scale, self.merge_dims = palm, beta2_scale, merge_dims
         self._state_init = [dict() for _ in params]
         if param_ecc is not None:  # heavyball/chainable.py:2421-2444: the live parameter is narrowed at construction
             narrowed = []
@@ -206,10 +208,18 @@ class SOAPOracle:
     K_OLD = "mars_mars_old_grad_5"  # pinned by a trajectory written from the reference
     K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
 
+    def _view_shape(self, shape):
+        """heavyball/utils.py:3726-3742: without merge_dims the tensors are taken as they are."""
+        return merged_shape(shape, self.max_precond_dim) if self.merge_dims else list(shape)
+
     def step(self, grads):
         is_precond = should_update(self.inner_group, self.schedule)
         self.step_count = self.step_count + 1
         step = self.step_count
+        if self.palm:  # heads the chain (heavyball/chainable.py:2693-2694) and rewrites the group's betas
+            from . import first_order as fo
+
+            self.betas = fo.palm_betas(self.betas, step, self.beta2_scale)
         self.fired.append(bool(is_precond))
         lr = step_lr(self.lr, step, self.warmup_steps)
         todo_p, todo_u, todo_g, todo_i = [], [], [], []
@@ -234,12 +244,12 @@ class SOAPOracle:
             if g is None:
                 continue
             st = self.state[i]
-            u = updates[i].reshape(merged_shape(g.shape, self.max_precond_dim)).unsqueeze(0)  # merged view + the bucket dimension
+            u = updates[i].reshape(self._view_shape(g.shape)).unsqueeze(0)  # merged view + the bucket dimension
             if self.K_M not in st:  # first step: ZeroGuard + GeneralGuard init, no update (heavyball/chainable.py:372-377)
                 self._moment(st, self.K_M, u)
                 self._moment(st, self.K_V, u)
                 # heavyball/chainable.py:1235-1238: the initial factors come from the gradient, not from the (clipped) update
-                g0 = g.clone().reshape(merged_shape(g.shape, self.max_precond_dim)).unsqueeze(0)
+                g0 = g.clone().reshape(self._view_shape(g.shape)).unsqueeze(0)
                 st[self.K_GG], st[self.K_Q] = init_preconditioner(g0, self.max_precond_dim, self.precondition_1d)
                 continue
             Q, GG = st[self.K_Q], st[self.K_GG]

@@ -389,6 +389,10 @@ def make_soap():
     conv = [(12, 4, 3, 3), (8, 3, 6)]
     run_traj("soap_merge", heavyball.SOAP, dict(precondition_frequency=4, max_precond_dim=64), conv, torch.float32, 6)
     run_traj("soap_merge3d", heavyball.SOAP, dict(precondition_frequency=2, max_precond_dim=12), conv, torch.float32, 5)
+    # merge_dims=False: the parameters as they are, one factor per dimension ((12,4,3,3) has four)
+    run_traj("soap_no_merge", heavyball.SOAP, dict(merge_dims=False, precondition_frequency=4), conv, torch.float32, 6)
+    # palm: beta2 = 1 - step ** -beta2_scale heads the chain
+    run_traj("soap_palm", heavyball.SOAP, dict(palm=True, beta2_scale=0.7, precondition_frequency=3), shapes, torch.float32, 6)
 
 
 def make_checkpoints():

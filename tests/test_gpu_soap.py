@@ -450,10 +450,10 @@ def test_soap_narrow_storage_matches_oracle(kwargs, rounding):
                 assert torch.equal(opt.state[p][0][km], opt2.state[p2][0][km])
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(20))
 def test_random_soap_configurations_match_oracle(seed):
     """Seeded draws over SOAP's switches (MARS, caution, decay, max_precond_dim down to sizes that drop a side, precondition_1d,
-    the four clip kinds on the gradient and on the update) and shapes (matrices of aspect ratio at most 2, so that both
+    palm, merge_dims, the four clip kinds on the gradient and on the update) and shapes (matrices of aspect ratio at most 2, so that both
     factors have full rank by the first refresh and the refreshed basis is determined by the data; vectors; a stack that
     is merged), seven steps with two refreshes, the step to 5e-3 against the oracle."""
     import random
@@ -476,6 +476,10 @@ def test_random_soap_configurations_match_oracle(seed):
     if rnd.random() < 0.2:
         shapes.append(())
     rnd.shuffle(shapes)
+    if rnd.random() < 0.3:
+        kwargs.update(palm=True, beta2_scale=rnd.choice([0.6, 0.8]))
+    if rnd.random() < 0.3:
+        kwargs["merge_dims"] = False
     print("case", seed, kwargs, shapes, flush=True)
     _run_soap_vs_oracle(shapes, kwargs, 7, 5e-3)
 
