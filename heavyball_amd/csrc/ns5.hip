@@ -433,9 +433,9 @@ __global__ __launch_bounds__(256) void ns_norm_final_kernel(const PrepGroup grp)
   if (threadIdx.x == 0) {
     float nrm = __builtin_sqrtf((float)(lds[0] + lds[1] + lds[2] + lds[3]));
     float eps = grp.eps;
-    if (grp.bf16_update) {  // a bf16 tensor's norm and the clamp bound are bf16 values
-      nrm = bf16_to_f32(f32_to_bf16_rne(nrm));
-      eps = bf16_to_f32(f32_to_bf16_rne(eps));
+    if (grp.bf16_update) {  // a bf16 tensor's norm is a bf16 value; so is the clamp bound, except under the legacy schedule, whose
+      nrm = bf16_to_f32(f32_to_bf16_rne(nrm));  // division promotes both sides to fp32 first (heavyball/utils.py:1174-1179, :1190)
+      if (!ka->it[pi].legacy) eps = bf16_to_f32(f32_to_bf16_rne(eps));
     }
     ka->it[pi].norm[0] = __builtin_fmaxf(nrm, eps);  // G.norm().clamp(min=eps), heavyball/utils.py:555
   }
@@ -454,12 +454,15 @@ __device__ __forceinline__ uint32_t ns_round_one(float v, float nrm, int legacy,
   if (legacy == 2) return f32_to_bf16_rne(v / nrm);  // bf16 update buffer: the quotient is a bf16 value already (heavyball/utils.py:2348-2349)
   Rand8 r, r2;
   const int lane8 = (int)(flat & 7);
-  if (aligned) r = aligned[0];
-  else r = rng.octet(flat & ~int64_t(7), HB_STREAM_NS_INPUT);
-  if (legacy == 0) return sr_bf16(v / nrm, r.bits16(lane8));
+  if (legacy != 3) {
+    if (aligned) r = aligned[0];
+    else r = rng.octet(flat & ~int64_t(7), HB_STREAM_NS_INPUT);
+    if (legacy == 0) return sr_bf16(v / nrm, r.bits16(lane8));
+  }
   if (aligned) r2 = aligned[1];
   else r2 = rng.octet(flat & ~int64_t(7), HB_STREAM_NS_INPUT + 1);
-  const uint32_t h = sr_bf16(v, r.bits16(lane8));
+  // legacy on a bf16 update buffer (3): its first round is the identity, the fp32 quotient is rounded stochastically
+  const uint32_t h = legacy == 3 ? f32_to_bf16_rne(v) : sr_bf16(v, r.bits16(lane8));
   return sr_bf16(bf16_to_f32(h) / nrm, r2.bits16(lane8));
 }
 
@@ -471,7 +474,8 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
   const float* __restrict__ g = ka->it[pi].g;
   const int rows = ka->it[pi].rows, cols = ka->it[pi].cols, transpose = ka->it[pi].transpose;
   const int64_t flat_base = ka->it[pi].flat_base;
-  const int legacy = grp.bf16_update ? 2 : ka->it[pi].legacy;  // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input)
+  // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input), 3: bf16 input under the legacy schedule (one, after the division)
+  const int legacy = grp.bf16_update ? (ka->it[pi].legacy ? 3 : 2) : ka->it[pi].legacy;
   const Rng rng = grp.rng;
   __shared__ uint16_t tile[64][64 + 8];  // +8: rows 144 B apart, so the column reads below spread over the banks
   const float nrm = ka->it[pi].norm[0];
@@ -497,8 +501,8 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
         const float4 a = *reinterpret_cast<const float4*>(g + f0), b = *reinterpret_cast<const float4*>(g + f0 + 4);
         const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
         Rand8 rr[2];
-        if (legacy != 2) rr[0] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT);
-        if (legacy == 1) rr[1] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT + 1);
+        if (legacy < 2) rr[0] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT);
+        if (legacy & 1) rr[1] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT + 1);
 #pragma unroll
         for (int e = 0; e < 8; ++e) h[e] = ns_round_one(v[e], nrm, legacy, rng, flat_base + f0 + e, rr);
       } else {
@@ -670,7 +674,6 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
     if (flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE)) return set_error(HB_EINVAL, "%s: unknown flag bits", who);
     if (((flag_of(i) & HB_NS_BF16_UPDATE) != 0) != (bf16_update != 0))
       return set_error(HB_EINVAL, "%s: HB_NS_BF16_UPDATE must be set for every matrix of a call or for none", who);
-    if ((flag_of(i) & HB_NS_LEGACY) && bf16_update) return set_error(HB_EINVAL, "%s: the legacy schedule on a bf16 update is not built", who);
   }
   for (int i = 0; i < n_mats; ++i) {
     if (!g[i] || !out[i]) return set_error(HB_EINVAL, "%s: null matrix pointer at %d", who, i);

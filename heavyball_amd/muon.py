@@ -224,8 +224,6 @@ class Muon(HBOptimizer):
                 if gdts - {torch.float32, torch.bfloat16} or len(gdts) > 1:
                     raise NotImplementedError("Muon: gradients of one bucket must all be float32 or all bfloat16")
                 ns_flags = _lib.NS_BF16_UPDATE if gdts == {torch.bfloat16} else 0
-                if ns_flags and mode == "legacy_newtonschulz":
-                    raise NotImplementedError("Muon: the legacy Newton-Schulz schedule with bfloat16 gradients")
                 mats = []
                 for i, p, _ in items:
                     if p.dim() < 2:

@@ -239,7 +239,9 @@ int hb_momentum(void* momentum, void* momentum_corr, int32_t momentum_fmt, float
  * `legacy` is a set of flags: HB_NS_LEGACY selects the legacy variant; HB_NS_BF16_UPDATE says that the reference's update
  * buffer is bfloat16 (bf16 gradients): the norm, the normalised input and the scaled result are then bf16 values rounded to
  * nearest, as torch computes them on a bf16 tensor, and the input gets no stochastic round (heavyball/utils.py:555-556,
- * :2348-2349, :577, :808-809).  g and out stay fp32 buffers (holding bf16-representable values in that case).
+ * :2348-2349, :577, :808-809).  g and out stay fp32 buffers (holding bf16-representable values in that case).  Both flags
+ * together: the legacy variant's first round is then the identity and its division, done in fp32 against the bf16-rounded
+ * norm, keeps its stochastic round (stream HB_STREAM_NS_INPUT + 1; heavyball/utils.py:641-645, :1174-1179).
  */
 enum { HB_NS_LEGACY = 1, HB_NS_BF16_UPDATE = 2 };
 int hb_ns5_workspace_bytes(int64_t rows, int64_t cols, int64_t* bytes);

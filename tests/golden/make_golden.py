@@ -193,7 +193,18 @@ def make_ecc():
 
 
 # ------------------------------------------------------------------------------------------------------
-def run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale=1e-2, param_scale=0.02, none_grad_for=None):
+def run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale=1e-2, param_scale=0.02, none_grad_for=None, mode=None):
+    if mode is not None:  # heavyball.utils.zeroth_power_mode for the length of the run, recorded as meta/zeroth_power_mode
+        before, heavyball.utils.zeroth_power_mode = heavyball.utils.zeroth_power_mode, mode
+        try:
+            run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale, param_scale, none_grad_for)
+        finally:
+            heavyball.utils.zeroth_power_mode = before
+        path = os.path.join(HERE, f"traj_{name}.pt")
+        out = torch.load(path, weights_only=True)
+        out["meta/zeroth_power_mode"] = mode
+        torch.save(out, path)
+        return
     gen = torch.Generator().manual_seed(0)
     params = [torch.nn.Parameter(torch.randn(s, generator=gen) * param_scale) for s in shapes]
     for p in params:
@@ -357,6 +368,24 @@ def make_ns5():
     torch.save(out, os.path.join(HERE, "ns5.pt"))
 
 
+def make_legacy():
+    """zeroth_power_mode = "legacy_newtonschulz": square matrices take the single coefficient triple and its input rounding
+    (heavyball/utils.py:637-657, :790-795), with fp32 and with bf16 gradients; Newton-Schulz vectors on bf16 inputs."""
+    shapes = [(16, 16), (16,), (24, 8), (8, 8)]
+    run_traj("muon_legacy", heavyball.Muon, dict(weight_decay=0.01), shapes, torch.float32, 4, mode="legacy_newtonschulz")
+    run_traj("muon_legacy_bf16grad", heavyball.Muon, dict(storage_dtype="bfloat16"), shapes, torch.bfloat16, 4, mode="legacy_newtonschulz")
+    out = {}
+    gen = torch.Generator().manual_seed(11)
+    for name, shape in [("sq", (16, 16)), ("wide", (8, 32)), ("tall", (32, 8)), ("sq64", (64, 64))]:
+        G = (torch.randn(shape, generator=gen) * 1e-2).bfloat16()
+        out[f"{name}/G"] = G.clone()
+        with half_rounding():
+            out[f"{name}/ns5"] = heavyball.utils.zeropower_via_newtonschulz5(G.clone(), 5).clone()
+            if shape[0] == shape[1]:
+                out[f"{name}/legacy"] = heavyball.utils.legacy_zeropower_via_newtonschulz5(G.clone(), 5).clone()
+    torch.save(out, os.path.join(HERE, "ns5_bf16.pt"))
+
+
 def make_muon():
     shapes = [(8, 16), (16,), (24, 8), (4, 3, 6)]
     run_traj("muon_default", heavyball.Muon, dict(weight_decay=0.01), shapes, torch.float32, 4)
@@ -440,7 +469,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "switches", "ns5", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -461,6 +490,8 @@ if __name__ == "__main__":
         make_ns5()
     if "muon" in which:
         make_muon()
+    if "legacy" in which:
+        make_legacy()
     if "soap" in which:
         make_soap()
     if "ckpt" in which:

@@ -34,13 +34,14 @@ def run_ns5(G, legacy=False, rng_mode=_lib.RNG_HALF, seed=0, step=0, base=0, sca
     nbytes = ctypes.c_int64()
     _lib.check(L.hb_ns5_workspace_bytes(rows, cols, ctypes.byref(nbytes)))
     ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
-    g = G.to(DEV).contiguous()
+    g = G.to(DEV, torch.float32).contiguous()  # a bf16 input travels as fp32 values under HB_NS_BF16_UPDATE
     out = torch.empty_like(g)
     coeffs = muon.LEGACY_COEFFS if legacy else muon.NS_COEFFS
     arr = (ctypes.c_float * 15)(*ns_coeff_array(coeffs))
     if scale is None:
         scale = max(1, rows / cols) ** 0.5
-    _lib.check(L.hb_ns5(g.data_ptr(), out.data_ptr(), rows, cols, arr, int(legacy), 1e-7, scale, rng_mode, seed, step, base, ws.data_ptr(),
+    flags = int(legacy) | (_lib.NS_BF16_UPDATE if G.dtype == torch.bfloat16 else 0)
+    _lib.check(L.hb_ns5(g.data_ptr(), out.data_ptr(), rows, cols, arr, flags, 1e-7, scale, rng_mode, seed, step, base, ws.data_ptr(),
                         nbytes.value, None))
     torch.cuda.synchronize()
     return out.cpu()
@@ -142,6 +143,50 @@ def test_ns5_matches_reference_vectors(name):
         assert rel_fro(run_ns5(G, legacy=True, scale=1.0), d[f"{name}/legacy"]) < NS_TOL
 
 
+@pytest.mark.parametrize("name", ["sq", "wide", "tall", "sq64"])
+def test_ns5_on_bf16_inputs_matches_reference_vectors(name):
+    """HB_NS_BF16_UPDATE, alone and with the legacy schedule, against vectors the reference computed on bf16 tensors."""
+    d = torch.load(os.path.join(GOLDEN, "ns5_bf16.pt"), weights_only=True)
+    print("case", name, flush=True)
+    G = d[f"{name}/G"]
+    got = run_ns5(G, scale=1.0)
+    assert torch.equal(got, got.bfloat16().float()) and rel_fro(got, d[f"{name}/ns5"].float()) < NS_TOL
+    if f"{name}/legacy" in d:
+        got = run_ns5(G, legacy=True, scale=1.0)
+        assert torch.equal(got, got.bfloat16().float()) and rel_fro(got, d[f"{name}/legacy"].float()) < NS_TOL
+
+
+@pytest.mark.parametrize("legacy", [False, True])
+def test_ns5_bf16_input_rounding_is_the_oracles(legacy):
+    """The normalised bf16 input the kernel feeds its first product, read back through a one-iteration identity schedule
+    (a = 1, b = c = 0 makes an iteration return X): the default schedule rounds the bf16 quotient to nearest, the legacy one
+    rounds the fp32 quotient stochastically with stream NS_INPUT + 1."""
+    from oracle import philox
+    from oracle.ecc import stochastic_round
+    gen = torch.Generator().manual_seed(3)
+    G = (torch.randn(96, 96, generator=gen) * 1e-2).bfloat16()
+    L = _lib.lib()
+    nbytes = ctypes.c_int64()
+    _lib.check(L.hb_ns5_workspace_bytes(96, 96, ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
+    g = G.to(DEV, torch.float32).contiguous()
+    out = torch.empty_like(g)
+    arr = (ctypes.c_float * 15)(*([1.0, 0.0, 0.0] * 5))
+    flags = int(legacy) | _lib.NS_BF16_UPDATE
+    print("case", legacy, flush=True)
+    _lib.check(L.hb_ns5(g.data_ptr(), out.data_ptr(), 96, 96, arr, flags, 1e-7, 1.0, _lib.RNG_PHILOX, 9, 4, 640, ws.data_ptr(), nbytes.value, None))
+    torch.cuda.synchronize()
+    nrm = G.norm()  # a bf16 value
+    if legacy:
+        r = PhiloxRounding(9, step=4, base=[640])
+        want = stochastic_round(G.float() / nrm.float().clamp(min=1e-7), r.noise16(philox.STREAM_NS_INPUT + 1, 0, G.shape)).float()
+    else:
+        want = (G / nrm.clamp(min=1e-7)).float()
+    got = out.cpu()
+    assert (got != want).float().mean() < 2e-3  # the norm's summation order may move its bf16 rounding once in a while: then all differ
+    assert rel_fro(got, want) < 1e-2
+
+
 @pytest.mark.parametrize("shape", [(256, 256), (128, 384), (384, 128), (300, 200), (130, 515), (512, 2048), (2304, 768), (256, 9000), (9000, 200), (768, 50257)])
 @pytest.mark.parametrize("rounding", ["half", "philox"])
 def test_ns5_matches_oracle(shape, rounding):
@@ -192,7 +237,7 @@ def test_ns5_input_rounding_is_the_oracles():
 # ---------------------------------------------------------------------------------------------------------------
 # the Muon optimizer class end to end
 # ---------------------------------------------------------------------------------------------------------------
-def _muon_pair(shapes, kwargs, rounding="half", seed=21):
+def _muon_pair(shapes, kwargs, rounding="half", seed=21, mode="newtonschulz"):
     import heavyball_amd
     from tests import helpers as H
 
@@ -201,7 +246,7 @@ def _muon_pair(shapes, kwargs, rounding="half", seed=21):
     opt.rounding, opt.rng_seed = rounding, seed
     base = opt._buckets[0][0].slab.offsets_np.tolist()
     r = HalfRounding() if rounding == "half" else PhiloxRounding(seed, base=base)
-    orc = muon.MuonOracle([h.clone() for h in host], rounding=r, **kwargs)
+    orc = muon.MuonOracle([h.clone() for h in host], rounding=r, mode=mode, **kwargs)
     return host, params, opt, orc
 
 
@@ -272,20 +317,27 @@ def _random_muon_case(seed):
     if rnd.random() < 0.4:
         shapes.append((rnd.randint(2, 6), rnd.randint(2, 6), rnd.choice([8, 24, 31])))
     rnd.shuffle(shapes)
-    return kwargs, gdt, shapes, rnd.choice(["half", "philox"])
+    rounding = rnd.choice(["half", "philox"])
+    mode = "newtonschulz"
+    if rnd.random() < 0.35:  # the legacy schedule, which square matrices take (heavyball/utils.py:790-795)
+        mode = "legacy_newtonschulz"
+        shapes += [(rnd.choice([8, 64, 130, 256]),) * 2, (3, 6, 18)]
+    return kwargs, gdt, shapes, rounding, mode
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(40))
 def test_random_muon_configurations_match_oracle(seed):
     """Seeded draws over Muon's momentum forms, MARS, caution, decay, storage of the momentum and of the parameter, gradient
-    dtype and shapes (vectors, thin and tiny matrices, stacks): momentum, MARS' old gradient and their corrections bit for
+    dtype, the Newton-Schulz schedule and shapes (vectors, thin and tiny matrices, stacks): momentum, MARS' old gradient and their corrections bit for
     bit, vectors bit for bit, matrices to the Newton-Schulz tolerance on the step taken."""
     from oracle.ecc import EccTensor
     from tests import helpers as H
 
-    kwargs, gdt, shapes, rounding = _random_muon_case(seed)
-    print("case", seed, kwargs, gdt, shapes, rounding, flush=True)
-    host, params, opt, orc = _muon_pair(shapes, kwargs, rounding)
+    import heavyball_amd
+
+    kwargs, gdt, shapes, rounding, mode = _random_muon_case(seed)
+    print("case", seed, kwargs, gdt, shapes, rounding, mode, flush=True)
+    host, params, opt, orc = _muon_pair(shapes, kwargs, rounding, mode=mode)
     if kwargs.get("param_ecc"):
         for b in opt._buckets[0]:
             for i, p in enumerate(b.params):
@@ -302,7 +354,11 @@ def test_random_muon_configurations_match_oracle(seed):
         prev_o = [q.decode() if isinstance(q, EccTensor) else q.clone() for q in orc.params]
         for p, g in zip(params, grads):
             p.grad = g.to(DEV)
-        opt.step()
+        heavyball_amd.muon.zeroth_power_mode = mode
+        try:
+            opt.step()
+        finally:
+            heavyball_amd.muon.zeroth_power_mode = "newtonschulz"
         orc.step([g.clone() for g in grads])
         torch.cuda.synchronize()
         for i, p in enumerate(params):
@@ -367,7 +423,11 @@ def test_muon_matches_reference_trajectories():
         for k in range(1, d["meta/steps"] + 1):
             for i, p in enumerate(params):
                 p.grad = d[f"step{k}/g{i}"].clone().to(DEV)
-            opt.step()
+            heavyball_amd.muon.zeroth_power_mode = d.get("meta/zeroth_power_mode", "newtonschulz")
+            try:
+                opt.step()
+            finally:
+                heavyball_amd.muon.zeroth_power_mode = "newtonschulz"
             torch.cuda.synchronize()
             for i, p in enumerate(params):
                 mom = d[f"step{k}/state{i}/{opt.KEY}"]

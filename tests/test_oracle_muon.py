@@ -34,6 +34,21 @@ def test_newton_schulz_matches_reference_vectors(name):
     assert rel_fro(out, d[f"{name}/orthogonal_scaled"]) < 1e-2
 
 
+@pytest.mark.parametrize("name", ["sq", "wide", "tall", "sq64"])
+def test_newton_schulz_on_bf16_inputs_matches_reference_vectors(name):
+    """A bf16 update buffer: the norm and the normalised input are bf16 values, the input's stochastic round is the identity; the
+    legacy variant divides in fp32 and rounds that quotient stochastically (heavyball/utils.py:555-556, :641-645, :1174-1179)."""
+    d = torch.load(os.path.join(GOLDEN, "ns5_bf16.pt"), weights_only=True)
+    G = d[f"{name}/G"]
+    assert G.dtype == torch.bfloat16
+    half = torch.full(G.shape, 1 << 15, dtype=torch.int32)
+    out = muon.newton_schulz5(G.clone(), half)
+    assert out.dtype == torch.bfloat16 and rel_fro(out, d[f"{name}/ns5"]) < 1e-2
+    if f"{name}/legacy" in d:
+        out = muon.legacy_newton_schulz5(G.clone(), half, half)
+        assert out.dtype == torch.bfloat16 and rel_fro(out, d[f"{name}/legacy"]) < 1e-2
+
+
 def test_polar_factor_invariant():
     """The per-iteration schedule drives every singular value towards 1: the result is close to U V^T of the SVD and
     its singular values lie in a band around 1 (a wrong coefficient, sign or a transposed operand leaves them far off)."""
@@ -90,7 +105,8 @@ def test_muon_trajectory_matches_reference(path):
     if "betas" in kwargs:
         kwargs["betas"] = tuple(kwargs["betas"])
     n = len([k for k in d if k.startswith("init/p")])
-    orc = muon.MuonOracle([d[f"init/p{i}"].clone() for i in range(n)], rounding=HalfRounding(), **kwargs)
+    orc = muon.MuonOracle([d[f"init/p{i}"].clone() for i in range(n)], rounding=HalfRounding(),
+                          mode=d.get("meta/zeroth_power_mode", "newtonschulz"), **kwargs)
     for k in range(1, d["meta/steps"] + 1):
         orc.step([d[f"step{k}/g{i}"].clone() for i in range(n)])
         for i in range(n):
