@@ -100,8 +100,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   const bool fast_sqrt = a.eps >= 1e-18f;
 
   RawT<kE> rp[kGroups], rg[kGroups], rm[kGroups], rv[kGroups], ro[kGroups], rs[kGroups];
-  float gtail[kGroups][kE];
-  bool tail[kGroups];
+  bool tail[kGroups];  // the group's gradient came by element loads: rg[k].a holds fp32 values whatever the gradient's format
   // the loads of one group
   auto fetch = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
@@ -114,7 +113,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
       } else {  // last, partial run of a gradient that is not padded: element loads
         tail[k] = true;
 #pragma unroll
-        for (int j = 0; j < kE; ++j) gtail[k][j] = e + j < valid ? load_elem(gbase, gf, g0 + e + j) : 0.0f;
+        for (int j = 0; j < kE; ++j) rg[k].a[j] = e + j < valid ? f2u(load_elem(gbase, gf, g0 + e + j)) : 0u;
       }
       if (kAdopt) rm[k] = rp[k] = RawT<kE>{};
       if constexpr (kLazy) {  // primaries only
@@ -147,7 +146,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
     Noise<kE> rn_p{};  // noise of the parameter's rounding
     if (!FULL && tail[k]) {
 #pragma unroll
-      for (int j = 0; j < kE; ++j) g[j] = gtail[k][j];
+      for (int j = 0; j < kE; ++j) g[j] = u2f(rg[k].a[j]);
     } else {
       raw_decode<GF>(rg[k], gf, g);
     }
