@@ -85,10 +85,8 @@ __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs 
         }
       }
       if (!kCount) {
-        Raw w;
         Rand8 rn = pf != HB_FMT_F32 ? a.rng.octet(idx, HB_STREAM_PARAM) : Rand8{{0, 0, 0, 0}};
-        raw_encode<PF>(w, pf, p, rn);
-        raw_store<PF>(w, pf, a.param, a.param_corr, idx);
+        raw_put<PF>(pf, p, rn, a.param, a.param_corr, idx);
       }
     }
     if (kCount) {

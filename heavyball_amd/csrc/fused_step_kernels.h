@@ -215,17 +215,16 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
           }
         } else {
           const Noise<kE> rn_og = og_rounds ? a.rng.noise<kE>(idx, HB_STREAM_OLD_GRAD) : Noise<kE>{};
-          raw_encode<SF>(w, sf, og, rn_og);
+          raw_put<SF>(sf, og, rn_og, a.og, a.og_corr, idx);
         }
-        raw_store<SF>(w, sf, a.og, a.og_corr, idx);
+        if (kCopy && (FULL || !tail[k])) raw_store<SF>(w, sf, a.og, a.og_corr, idx);
         if (write_grad) {
 #pragma unroll
           for (int j = 0; j < kE; ++j)
             if (FULL || e + j < valid) store_elem(const_cast<char*>(gbase), gf, g0 + e + j, g[j]);
         }
         if (mars_only) {
-          raw_encode<HB_FMT_F32>(w, HB_FMT_F32, g, Noise<kE>{});
-          raw_store<HB_FMT_F32>(w, HB_FMT_F32, a.param, nullptr, idx);
+          raw_put<HB_FMT_F32>(HB_FMT_F32, g, Noise<kE>{}, a.param, nullptr, idx);
           return;
         }
       }
@@ -301,27 +300,21 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
 #pragma unroll
         for (int j = 0; j < kE; ++j) p[j] = p[j] * a.omdl + u[j] * a.neg_lr;  // heavyball/utils.py:2389
       }
-      RawT<kE> w;
       Noise<kE> rn_m{}, rn_v{};  // exp_avg and exp_avg_sq share their Philox calls
       if (state_rounds) a.rng.noise_pair<kE>(idx, HB_STREAM_EXP_AVG >> 1, rn_m, rn_v);
       if (!kAdopt || !warmup) {
-        raw_encode<SF>(w, sf, m, rn_m);
-        raw_store<SF>(w, sf, a.m, a.m_corr, idx);
+        raw_put<SF>(sf, m, rn_m, a.m, a.m_corr, idx);
       }
-      raw_encode<SF>(w, sf, v, rn_v);
-      raw_store<SF>(w, sf, a.v, a.v_corr, idx);
+      raw_put<SF>(sf, v, rn_v, a.v, a.v_corr, idx);
       if (kMix) {
         const Noise<kE> rn = state_rounds ? a.rng.noise<kE>(idx, HB_STREAM_EXP_AVG_SLOW) : Noise<kE>{};
-        raw_encode<SF>(w, sf, sl, rn);
-        raw_store<SF>(w, sf, a.s3, a.s3_corr, idx);
+        raw_put<SF>(sf, sl, rn, a.s3, a.s3_corr, idx);
       }
       if (update_only && a.upd != nullptr) {
-        raw_encode<HB_FMT_F32>(w, HB_FMT_F32, p, Noise<kE>{});
-        raw_store<HB_FMT_F32>(w, HB_FMT_F32, a.upd, nullptr, idx);
+        raw_put<HB_FMT_F32>(HB_FMT_F32, p, Noise<kE>{}, a.upd, nullptr, idx);
       } else if (!kAdopt || !warmup) {
         if (!MARS && pf != HB_FMT_F32) rn_p = a.rng.noise<kE>(idx, HB_STREAM_PARAM);
-        raw_encode<PF>(w, pf, p, rn_p);
-        raw_store<PF>(w, pf, a.param, a.param_corr, idx);
+        raw_put<PF>(pf, p, rn_p, a.param, a.param_corr, idx);
       }
     }
   };

@@ -33,7 +33,12 @@ __device__ __forceinline__ uint32_t f32_to_f16_rne(float x) { return (uint32_t)_
 // ---------------------------------------------------------------------------------------------------------
 struct Rand8 {  // the four words of one call; also: the noise of an octet for one stream (two calls, see Rng::octet)
   uint32_t w[4];
-  __device__ __forceinline__ uint32_t bits16(int j) const { return (w[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu; }
+  // selects instead of an indexed read: with a run-time j an indexed array would live in scratch memory
+  __device__ __forceinline__ uint32_t bits16(int j) const {
+    const int k = j >> 1;
+    const uint32_t x = k == 0 ? w[0] : k == 1 ? w[1] : k == 2 ? w[2] : w[3];
+    return (x >> ((j & 1) * 16)) & 0xFFFFu;
+  }
 };
 // noise of E consecutive elements for one stream: 16 bits each, element j in word j >> 1
 template <int E>
@@ -455,6 +460,24 @@ __device__ __forceinline__ void raw_store(const RawT<E>& r, int f, char* prim, c
 #define HB_CALL(X) raw_store_s<X, E>(r, prim, corr, idx)
   HB_FMT_SWITCH(F, f, HB_CALL);
 #undef HB_CALL
+}
+// encode + store in one dispatch: the packed words live inside one case of the switch.  (Shared between an encode switch and
+// a store switch they are written and read with a different type in every case, and the compiler then keeps them in scratch
+// memory.)
+template <int F, int E>
+__device__ __forceinline__ void raw_put(int f, const float (&x)[E], const Noise<E>& rnd, char* prim, char* corr, int64_t idx) {
+#define HB_CALL(X)                     \
+  do {                                 \
+    RawT<E> r_;                        \
+    raw_encode_s<X, E>(r_, x, rnd);    \
+    raw_store_s<X, E>(r_, prim, corr, idx); \
+  } while (0)
+  HB_FMT_SWITCH(F, f, HB_CALL);
+#undef HB_CALL
+}
+template <int F>
+__device__ __forceinline__ void raw_put(int f, const float (&x)[8], const Rand8& rnd, char* prim, char* corr, int64_t idx) {
+  raw_put<F, 8>(f, x, Noise<8>{{rnd.w[0], rnd.w[1], rnd.w[2], rnd.w[3]}}, prim, corr, idx);
 }
 // octet kernels hand their noise over as the four words of a Rand8
 template <int F>

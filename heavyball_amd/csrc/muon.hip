@@ -71,11 +71,8 @@ __global__ __launch_bounds__(kMThreads) void momentum_kernel(char* __restrict__ 
       const bool state_rounds = MF == kDyn;  // bf16 storage rounds stochastically, ECC pairs draw their correction
       const Rand8 rn_m = state_rounds ? rng.octet(idx, HB_STREAM_EXP_AVG) : Rand8{{0, 0, 0, 0}};
       const Rand8 none{{0, 0, 0, 0}};
-      Raw w;
-      raw_encode<MF>(w, mf, m, rn_m);
-      raw_store<MF>(w, mf, mom, mom_corr, idx);
-      raw_encode<HB_FMT_F32>(w, 0, u, none);
-      raw_store<HB_FMT_F32>(w, 0, reinterpret_cast<char*>(upd), nullptr, idx);
+      raw_put<MF>(mf, m, rn_m, mom, mom_corr, idx);
+      raw_put<HB_FMT_F32>(0, u, none, reinterpret_cast<char*>(upd), nullptr, idx);
     }
   }
 }

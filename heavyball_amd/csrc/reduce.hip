@@ -98,8 +98,7 @@ __global__ __launch_bounds__(kRThreads) void scale_kernel(float* __restrict__ x,
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] *= s;
         Rand8 none{{0, 0, 0, 0}};
-        raw_encode<HB_FMT_F32>(r, 0, v, none);
-        raw_store<HB_FMT_F32>(r, 0, reinterpret_cast<char*>(x), nullptr, flat0 + e);
+        raw_put<HB_FMT_F32>(0, v, none, reinterpret_cast<char*>(x), nullptr, flat0 + e);
       }
     }
   }
