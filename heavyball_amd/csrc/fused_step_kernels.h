@@ -203,21 +203,26 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
         g[j] = gc;
       }
       if (!kCount) {
-        RawT<kE> w;
         // a bf16 gradient stored into a bf16 primary is its own encoding: the primary takes the gradient's bits and the
         // correction is zero (what the encoder would compute: the residual is 0 and floor(0 + noise / 65536) = 0)
         constexpr bool kCopy = GF == HB_FMT_BF16 && (SF == HB_FMT_BF16 || SF == HB_FMT_ECC_BF16_8 || SF == HB_FMT_ECC_BF16_16);
-        if (kCopy && (FULL || !tail[k])) {
+        if constexpr (kCopy) {  // a compiled-in format: one store behind both ways of filling the words
+          RawT<kE> w;
+          if (FULL || !tail[k]) {
 #pragma unroll
-          for (int i = 0; i < kE / 2; ++i) {
-            w.a[i] = rg[k].a[i];
-            w.c[i] = 0;
+            for (int i = 0; i < kE / 2; ++i) {
+              w.a[i] = rg[k].a[i];
+              w.c[i] = 0;
+            }
+          } else {
+            const Noise<kE> rn_og = og_rounds ? a.rng.noise<kE>(idx, HB_STREAM_OLD_GRAD) : Noise<kE>{};
+            raw_encode<SF>(w, sf, og, rn_og);
           }
+          raw_store<SF>(w, sf, a.og, a.og_corr, idx);
         } else {
           const Noise<kE> rn_og = og_rounds ? a.rng.noise<kE>(idx, HB_STREAM_OLD_GRAD) : Noise<kE>{};
           raw_put<SF>(sf, og, rn_og, a.og, a.og_corr, idx);
         }
-        if (kCopy && (FULL || !tail[k])) raw_store<SF>(w, sf, a.og, a.og_corr, idx);
         if (write_grad) {
 #pragma unroll
           for (int j = 0; j < kE; ++j)
