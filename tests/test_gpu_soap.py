@@ -307,6 +307,17 @@ def test_soap_mid_size_own_eigh_signed_momentum():
     assert sum(orc.fired) == 2  # the float-accumulated schedule of frequency 3 fires at steps 3 and 7
 
 
+@pytest.mark.timeout(400)
+def test_soap_at_benchmark_shapes_matches_oracle():
+    """The three matrices of the SOAP benchmark configuration ([2048, 2048], [2048, 8192], [8192, 2048]) under the default
+    max_precond_dim (the 8192-wide sides get no factor, four 2048-wide ones remain): initialisation, a step, a step with a
+    refresh (the batched factorisation of four bases at once) and a step in the refreshed basis, the checker's basis adopted
+    after the first step, every step to 5e-3.  The checker needs about half a minute of CPU time."""
+    shapes = [(2048, 2048), (2048, 8192), (8192, 2048)]
+    opt, orc = _run_soap_vs_oracle(shapes, dict(precondition_frequency=3), 4, 5e-3)
+    assert orc.fired == [False, False, True, False]
+
+
 def test_soap_matches_oracle_with_refresh():
     """frequency 4: the eigenbasis is refreshed at steps 4, 8: exercises power iteration + QR + the rotation of exp_avg.
     Shapes are chosen so that both factors have full rank by the first refresh (4 gradients): QR of a power-iteration step
