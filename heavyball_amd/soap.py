@@ -10,6 +10,9 @@ refreshed with one power-iteration step + a QR factorisation when the schedule f
 Householder's up to column signs, which the step is invariant to) and falls back to ``torch.linalg.qr`` when a factor is
 numerically rank-deficient; ``eigh`` stays in torch.
 
+With ``split`` a parameter larger than max_precond_dim in some dimension is preconditioned block by block, every block with a
+state of its own under ``state[p][k]`` (heavyball/utils.py:274-286, :1612-1623).
+
 State layout of the reference: ``scale_by_soap_exp_avg_2`` / ``scale_by_soap_exp_avg_sq_2`` with a leading bucket
 dimension of 1, ``scale_by_soap_Q_3`` / ``scale_by_soap_GG_3`` as lists with one ``[1, d, d]`` tensor (or None) per dimension.
 """
@@ -43,6 +46,25 @@ def merged_shape(shape, max_precond_dim: int):
     if cum > 1:
         new_shape.append(cum)
     return [shape[0], *new_shape[::-1]] if len(shape) else []
+
+
+def split_blocks(shape, max_precond_dim: int):
+    """heavyball/utils.py:274-286 (``dim_merger`` with split=True) as index arithmetic: None when no dimension of the merged view
+    exceeds max_precond_dim, else one ``(slices into the merged view, shape of the block)`` per block.  Every oversized dimension is
+    cut into runs of max_precond_dim (the last one shorter); the blocks are ordered with the cuts of the last such dimension
+    outermost; dimensions of size one in the merged view are dropped from a block, whose remaining shape is merged again."""
+    import itertools
+
+    merged = merged_shape(shape, max_precond_dim) if len(shape) else []
+    cuts = [[(a, min(a + max_precond_dim, sh)) for a in range(0, sh, max_precond_dim)] if sh > max_precond_dim else [(0, sh)] for sh in merged]
+    if all(len(c) == 1 for c in cuts):
+        return None
+    out = []
+    for combo in itertools.product(*reversed(cuts)):
+        spans = combo[::-1]  # back in dimension order
+        kept = [b - a for (a, b), sh in zip(spans, merged) if sh != 1]
+        out.append((tuple(slice(a, b) for a, b in spans), merged_shape(kept, max_precond_dim) if kept else []))
+    return out
 
 
 class _Gemm:
@@ -134,13 +156,18 @@ class SOAP(HBOptimizer):
         del defaults["precond_scheduler"]
         self.precond_schedule = 1 / defaults.pop("precondition_frequency")  # heavyball/__init__.py:842-858
         # precond_grad_accum is read by PSGD's guard only (heavyball/chainable.py:304-345): SOAP's chain ignores it, and so does this
-        if split:
-            raise NotImplementedError("SOAP on the HIP kernels: split (one state per block of a parameter) is not built")
+        if split and merge_dims and (mars or caution or param_ecc or ecc or storage_dtype != "float32"):
+            # one state per block (heavyball/utils.py:274-286, :1612-1623): built for the preconditioner's own state in fp32; state
+            # outside it (MARS' old gradient), narrow storage and the per-block count of caution are not
+            raise NotImplementedError("SOAP on the HIP kernels: split together with mars, caution, ecc, param_ecc or non-fp32 storage")
         if mars and (ecc or storage_dtype != "float32"):
             raise NotImplementedError("SOAP on the HIP kernels: mars together with ecc or non-fp32 storage")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
         if mars and self.gradient_clipping is not None:
             raise NotImplementedError("SOAP on the HIP kernels: mars together with gradient_clipping")
+        per_tensor = ("l2_clip_", "rmsnorm_clip_")
+        if split and merge_dims and (self.gradient_clipping in per_tensor or self.update_clipping in per_tensor):
+            raise NotImplementedError("SOAP on the HIP kernels: split together with clipping by a norm per tensor (per block in the reference)")
 
     def _run_group(self, gi, group, active):
         active = [(p, g) for p, g in active if p.numel() > 0]  # an empty tensor has nothing to precondition or update
@@ -205,13 +232,9 @@ class SOAP(HBOptimizer):
             stream = current_stream_ptr(b.device)
             updated, keep, refresh = [], [], []
             with torch.cuda.device(b.device):
-                for (i, p, g), g32 in zip(items, raw[key]):
-                    keep.append(g32)
-                    # heavyball/utils.py:3726-3742: without merge_dims the parameter is taken as it is
-                    shape = (merged_shape(p.shape, max_dim) if group.get("merge_dims", True) else list(p.shape)) if p.dim() > 0 else []
-                    G0 = g32.reshape(shape) if shape else g32.reshape(1)  # the gradient
-                    G = b.slab.view("_clip", i).reshape(G0.shape) if self.gradient_clipping is not None else G0  # the update
-                    st = self._state0(p)
+                def precondition(st, G0, G, out, base):
+                    """One tensor or block: G0 the gradient, G the update that goes through the preconditioner, both in the merged
+                    view; the preconditioned update lands in ``out``.  False on the first step, which only initialises."""
                     if K_M not in st:  # first step: initialise, no update (heavyball/chainable.py:372-377, utils.py:1362-1388)
                         for km in (K_M, K_V):  # zero_guard with the group's storage (heavyball/chainable.py:277-301)
                             st[km] = torch.zeros((1, *G.shape), dtype=mom_prim, device=b.device)
@@ -239,9 +262,8 @@ class SOAP(HBOptimizer):
                             Q.append(torch.flip(vec, [-1]).to(torch.float32).contiguous())
                         st[K_GG], st[K_Q] = GG, Q
                         st.setdefault("is_initialized", set()).update({0, 2, 3})
-                        continue
+                        return False
                     Q, GG = st[K_Q], st[K_GG]
-                    out = b.slab.view("_update", i).view(G.shape)
                     gp = self._project(gemm, G, Q, back=False)
                     a1, oma1 = debiased_weights(beta1, adam_step)
                     a2, oma2 = debiased_weights(beta2, adam_step)
@@ -253,7 +275,6 @@ class SOAP(HBOptimizer):
                     _lib.check(L.hb_adam_precond(m32.data_ptr(), v32.data_ptr(), gp.data_ptr(), gp.data_ptr(), gp.numel(), a1, oma1,
                                                  a2, oma2, float(f32(group["eps"])), stream), "hb_adam_precond")  # fmt: skip
                     if mom_fmt != _lib.FMT_F32:
-                        base = int(b.slab.offsets_np[i])
                         self._narrow(L, st, K_M, m32, mom_fmt, _lib.STREAM_EXP_AVG, step, base, stream)
                         self._narrow(L, st, K_V, v32, mom_fmt, _lib.STREAM_EXP_AVG_SQ, step, base, stream)
                     back = self._project(gemm, gp, Q, back=True, out=out)
@@ -267,8 +288,35 @@ class SOAP(HBOptimizer):
                         if mom_fmt == _lib.FMT_F32:
                             refresh.append((GG, Q, st[K_M]))
                         else:  # the rotation reads exp_avg as stored (heavyball/utils.py:883) and writes it back through the codec
-                            refresh.append((GG, Q, self._widen(L, st, K_M, mom_fmt, stream), st, int(b.slab.offsets_np[i])))
-                    updated.append(i)
+                            refresh.append((GG, Q, self._widen(L, st, K_M, mom_fmt, stream), st, base))
+                    return True
+
+                for (i, p, g), g32 in zip(items, raw[key]):
+                    keep.append(g32)
+                    # heavyball/utils.py:3726-3742: without merge_dims the parameter is taken as it is
+                    merging = group.get("merge_dims", True)
+                    shape = (merged_shape(p.shape, max_dim) if merging else list(p.shape)) if p.dim() > 0 else []
+                    G0 = g32.reshape(shape) if shape else g32.reshape(1)  # the gradient
+                    G = b.slab.view("_clip", i).reshape(G0.shape) if self.gradient_clipping is not None else G0  # the update
+                    out = b.slab.view("_update", i).view(G.shape)
+                    blocks = split_blocks(p.shape, max_dim) if merging and group.get("split") and p.dim() > 0 else None
+                    if blocks is None:
+                        if precondition(self._state0(p), G0, G, out, int(b.slab.offsets_np[i])):
+                            updated.append(i)
+                        continue
+                    # split: every block is preconditioned on its own, with its own state (heavyball/utils.py:274-286, :1612-1623);
+                    # a block is a strided part of the parameter, so it is gathered, and its update scattered into the slab
+                    done = False
+                    for k, (where, bshape) in enumerate(blocks):
+                        bshape = bshape or [1]
+                        g0b = G0[where].contiguous().reshape(bshape)
+                        gb = g0b if G is G0 else G[where].contiguous().reshape(bshape)
+                        ob = torch.empty_like(gb)
+                        if precondition(self.state[p].setdefault(k, {}), g0b, gb, ob, 0):
+                            out[where].copy_(ob.reshape(out[where].shape))
+                            done = True
+                    if done:
+                        updated.append(i)
                 if refresh:
                     self._refresh(gemm, refresh)
                     for job in refresh:
@@ -303,16 +351,23 @@ class SOAP(HBOptimizer):
 
     def _rehome_state(self):
         """torch's ``load_state_dict`` casts floating-point state to the parameter's dtype: the moments go back to their storage
-        dtype (their values are representable there, heavyball/chainable.py:2452-2484 does the same)."""
+        dtype (their values are representable there, heavyball/chainable.py:2452-2484 does the same).  A tensor that needs no
+        cast is handed over as it is, so a state_dict taken from a live optimizer in the same process would share its moments,
+        factors and bases with this one: every state tensor of the preconditioner is copied."""
         super()._rehome_state()
         for group in self.param_groups:
             for p in group["params"]:
-                st = self.state.get(p, {}).get(0) if p in self.state else None
-                if not isinstance(st, dict):
+                if p not in self.state:
                     continue
-                for key in (K_M, K_V, K_M + "::ecc", K_V + "::ecc"):
-                    if isinstance(st.get(key), torch.Tensor):
-                        st[key] = st[key].to(self._role_dtype(group, key)).contiguous()
+                for st in self.state[p].values():  # block 0, and the further blocks of a split parameter
+                    if not isinstance(st, dict):
+                        continue
+                    for key in (K_M, K_V, K_M + "::ecc", K_V + "::ecc"):
+                        if isinstance(st.get(key), torch.Tensor):
+                            st[key] = st[key].to(self._role_dtype(group, key), copy=True).contiguous()
+                    for key in (K_Q, K_GG):
+                        if isinstance(st.get(key), (list, tuple)):
+                            st[key] = [None if t is None else t.to(torch.float32, copy=True).contiguous() for t in st[key]]
 
     # -- pieces ----------------------------------------------------------------------------------------------------
     def _widen(self, L, st, key, fmt, stream):

@@ -50,6 +50,33 @@ def merged_shape(shape, max_precond_dim: int):
     return [shape[0], *new_shape[::-1]]
 
 
+def dim_merger(t: Tensor, max_precond_dim: int, split: bool):
+    """heavyball/utils.py:240-286 on a tensor: the merged view; with ``split`` every dimension larger than max_precond_dim is
+    cut into blocks of at most that size (the blocks of the last such dimension outermost in the order), dimensions of size
+    one are dropped from the blocks, and each block is merged again.  A tensor that needs no cut comes back as the merged view."""
+    new = t.reshape(merged_shape(t.shape, max_precond_dim))
+    if not split:
+        return new
+    blocks = [new]
+    for i, sh in reversed(list(enumerate(new.shape))):
+        if sh == 1:
+            blocks = [b.squeeze(dim=i) for b in blocks]
+            continue
+        if sh <= max_precond_dim:
+            continue
+        blocks = [a for b in blocks for a in b.split(max_precond_dim, dim=i)]
+    if len(blocks) == 1:
+        return new
+    out = []
+    for b in blocks:
+        r = dim_merger(b, max_precond_dim, split)
+        if isinstance(r, list):
+            out.extend(r)
+        else:
+            out.append(r)
+    return out
+
+
 def update_ggt(grad: Tensor, GG: List[Optional[Tensor]], max_precond_dim: int, precondition_1d: bool, beta):
     """heavyball/utils.py:1205-1221: GG_i <- GG_i * (1 - a) + (contraction of grad with itself over all but dim i) * a, a = 1 - beta."""
     if grad.dim() == 2 and (not precondition_1d or grad.shape[1] > max_precond_dim):
@@ -153,13 +180,15 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
 
 
 class SOAPOracle:
-    """heavyball.SOAP (heavyball/__init__.py:861-909) with split=False."""
+    """heavyball.SOAP (heavyball/__init__.py:861-909).  With ``split`` a parameter larger than max_precond_dim in some dimension is
+    preconditioned block by block (heavyball/utils.py:274-286, :1612-1623): every block has its own state, ``state[i]`` holding
+    that of block 0 and ``block_state[i][k]`` that of block k >= 1."""
 
     def __init__(self, params, lr=3e-3, betas=(0.9, 0.95), shampoo_beta=0.95, eps=1e-8, weight_decay=0.01, precondition_frequency=2,
                  max_precond_dim=2048, precondition_1d=False, warmup_steps=0, gradient_clipping=None,
                  update_clipping=None, mars=False, mars_gamma=0.0025, ecc=None, storage_dtype="float32", param_ecc=None,
                  caution=False, cautious_weight_decay=False, precond_grad_accum=False, palm=False, beta2_scale=0.8, merge_dims=True,
-                 rounding=None):  # fmt: skip
+                 split=False, rounding=None):  # fmt: skip
         from . import philox
         from .ecc import MODES, EccTensor
         from .rounding import HalfRounding
@@ -171,6 +200,11 @@ class SOAPOracle:
         self.param_ecc = param_ecc
         self.mars, self.mars_gamma = mars, mars_gamma
         self.palm, self.beta2_scale, self.merge_dims = palm, beta2_scale, merge_dims
+        self.split = split and merge_dims  # heavyball/utils.py:3726-3728: without merge_dims nothing is merged or cut
+        if self.split and (mars or param_ecc is not None or gradient_clipping in ("l2_clip_", "rmsnorm_clip_")
+                           or update_clipping in ("l2_clip_", "rmsnorm_clip_")):  # fmt: skip
+            raise NotImplementedError("split with state or norms per block outside the preconditioner")
+        self.block_state = [dict() for _ in params]
         self._state_init = [dict() for _ in params]
         if param_ecc is not None:  # heavyball/chainable.py:2421-2444: the live parameter is narrowed at construction
             narrowed = []
@@ -243,29 +277,35 @@ class SOAPOracle:
         for i, (p, g) in enumerate(zip(self.params, grads)):
             if g is None:
                 continue
-            st = self.state[i]
-            u = updates[i].reshape(self._view_shape(g.shape)).unsqueeze(0)  # merged view + the bucket dimension
-            if self.K_M not in st:  # first step: ZeroGuard + GeneralGuard init, no update (heavyball/chainable.py:372-377)
-                self._moment(st, self.K_M, u)
-                self._moment(st, self.K_V, u)
-                # heavyball/chainable.py:1235-1238: the initial factors come from the gradient, not from the (clipped) update
-                g0 = g.clone().reshape(self._view_shape(g.shape)).unsqueeze(0)
-                st[self.K_GG], st[self.K_Q] = init_preconditioner(g0, self.max_precond_dim, self.precondition_1d)
-                continue
-            Q, GG = st[self.K_Q], st[self.K_GG]
-            gp = project(u, Q, False)
-            rounding = self.rounding.at_step(int(step))
-            m_st, v_st = self._moment(st, self.K_M, u), self._moment(st, self.K_V, u)
-            precond = adam_(m_st, v_st, gp, self.betas[0], self.betas[1], step - 1, self.eps, rounding, i)
-            precond = project(precond, Q, True)
-            beta = beta_debias(self.shampoo_beta, step)  # heavyball/chainable.py:1244
-            update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta)
-            if is_precond:
-                refresh_basis(GG, Q, m_st, rounding, i)
-            todo_p.append(p)
-            todo_u.append(precond.squeeze(0).reshape(p.shape))
-            todo_g.append(g)
-            todo_i.append(i)
+            if self.split:  # blocks of the parameter, of the gradient and of the update, cut alike
+                pv, gv, uv = (dim_merger(t, self.max_precond_dim, True) for t in (p, g, updates[i]))
+                blocks = list(zip(pv, gv, uv)) if isinstance(pv, list) else [(p, g, updates[i])]
+            else:
+                blocks = [(p, g, updates[i])]
+            for k, (p, g, upd) in enumerate(blocks):
+                st = self.state[i] if k == 0 else self.block_state[i].setdefault(k, {})
+                u = upd.reshape(self._view_shape(g.shape)).unsqueeze(0)  # merged view + the bucket dimension
+                if self.K_M not in st:  # first step: ZeroGuard + GeneralGuard init, no update (heavyball/chainable.py:372-377)
+                    self._moment(st, self.K_M, u)
+                    self._moment(st, self.K_V, u)
+                    # heavyball/chainable.py:1235-1238: the initial factors come from the gradient, not from the (clipped) update
+                    g0 = g.clone().reshape(self._view_shape(g.shape)).unsqueeze(0)
+                    st[self.K_GG], st[self.K_Q] = init_preconditioner(g0, self.max_precond_dim, self.precondition_1d)
+                    continue
+                Q, GG = st[self.K_Q], st[self.K_GG]
+                gp = project(u, Q, False)
+                rounding = self.rounding.at_step(int(step))
+                m_st, v_st = self._moment(st, self.K_M, u), self._moment(st, self.K_V, u)
+                precond = adam_(m_st, v_st, gp, self.betas[0], self.betas[1], step - 1, self.eps, rounding, i)
+                precond = project(precond, Q, True)
+                beta = beta_debias(self.shampoo_beta, step)  # heavyball/chainable.py:1244
+                update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta)
+                if is_precond:
+                    refresh_basis(GG, Q, m_st, rounding, i)
+                todo_p.append(p)
+                todo_u.append(precond.squeeze(0).reshape(p.shape))
+                todo_g.append(g)
+                todo_i.append(i)
         if todo_p and self.update_clipping is not None:  # heavyball/chainable.py:2700-2701
             from . import first_order as fo
 

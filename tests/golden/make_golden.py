@@ -55,11 +55,13 @@ def hexf(t):
 
 
 def flat_state(opt, p):
+    """The state of a parameter under its plain keys; the states of the further blocks of a split parameter
+    (heavyball/utils.py:1612-1623: one state per view) under ``block<k>/<key>``."""
     out = {}
     for idx, st in opt.state[p].items():
         if isinstance(st, dict):
             for k, v in st.items():
-                out[k] = v
+                out[k if idx == 0 else f"block{idx}/{k}"] = v
     return out
 
 
@@ -420,6 +422,10 @@ def make_soap():
     run_traj("soap_merge3d", heavyball.SOAP, dict(precondition_frequency=2, max_precond_dim=12), conv, torch.float32, 5)
     # merge_dims=False: the parameters as they are, one factor per dimension ((12,4,3,3) has four)
     run_traj("soap_no_merge", heavyball.SOAP, dict(merge_dims=False, precondition_frequency=4), conv, torch.float32, 6)
+    # split: every dimension above max_precond_dim is cut into blocks, each block preconditioned with a state of its own:
+    # (20,12) -> six blocks, (16,) -> two vectors, (6,30) -> four blocks
+    run_traj("soap_split", heavyball.SOAP, dict(split=True, max_precond_dim=8, precondition_frequency=3, weight_decay=0.1),
+             [(20, 12), (16,), (6, 30)], torch.float32, 6)  # fmt: skip
     # palm: beta2 = 1 - step ** -beta2_scale heads the chain
     run_traj("soap_palm", heavyball.SOAP, dict(palm=True, beta2_scale=0.7, precondition_frequency=3), shapes, torch.float32, 6)
 

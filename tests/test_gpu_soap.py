@@ -3,6 +3,7 @@ float64 matmul, 1e-6 relative), the Adam-in-the-rotated-basis kernel (bit-exact 
 optimizer end to end against the CPU oracle and the trajectories recorded from the reference."""
 
 import glob
+import io
 import json
 import os
 
@@ -223,9 +224,11 @@ def _adopt_basis(opt, params, basis_of):
     so the vectors spanning its null space are an arbitrary choice of the LAPACK implementation, and Adam in the rotated
     basis is not invariant to that choice. For a comparison over later steps the test takes the checker's choice."""
     for i, p in enumerate(params):
-        for li, q in enumerate(opt.state[p][0]["scale_by_soap_Q_3"]):
-            if q is not None:
-                q.copy_(basis_of(i, li))
+        for k, st in opt.state[p].items():  # block 0, and the further blocks of a split parameter
+            if isinstance(st, dict) and "scale_by_soap_Q_3" in st:
+                for li, q in enumerate(st["scale_by_soap_Q_3"]):
+                    if q is not None:
+                        q.copy_(basis_of(i, li, k))
 
 
 def _run_soap_vs_oracle(shapes, kwargs, steps, tol, adopt=True, grad_fn=None, signed=False, diag_tol=1e-4):
@@ -283,7 +286,7 @@ def _run_soap_vs_oracle(shapes, kwargs, steps, tol, adopt=True, grad_fn=None, si
                 if gg is not None:
                     assert rel_fro(st[orc.K_GG][li], gg) < 1e-5
         if k == 1 and adopt:
-            _adopt_basis(opt, params, lambda i, li: orc.state[i][orc.K_Q][li].to(DEV))
+            _adopt_basis(opt, params, lambda i, li, k: (orc.state[i] if k == 0 else orc.block_state[i][k])[orc.K_Q][li].to(DEV))
     return opt, orc
 
 
@@ -363,7 +366,7 @@ def test_soap_matches_reference_trajectories():
             opt.step()
             torch.cuda.synchronize()
             if k == 1:
-                _adopt_basis(opt, params, lambda i, li: d[f"step1/state{i}/scale_by_soap_Q_3/{li}"].to(DEV))
+                _adopt_basis(opt, params, lambda i, li, k: d[f"step1/state{i}/" + (f"block{k}/" if k else "") + f"scale_by_soap_Q_3/{li}"].to(DEV))
             for i, p in enumerate(params):
                 want, got = d[f"step{k}/p{i}"], p.detach().cpu()
                 ck = f"step{k}/state{i}/param::ecc"
@@ -381,6 +384,20 @@ def test_soap_matches_reference_trajectories():
                     gk = f"step{k}/state{i}/scale_by_soap_GG_3/{li}"
                     if gk in d:
                         assert torch.allclose(opt.state[p][0]["scale_by_soap_GG_3"][li].cpu(), d[gk], rtol=1e-4, atol=1e-8)
+                # a split parameter: one state per block, in the reference's order
+                blocks = {int(kk.split("/")[2][5:]) for kk in d if kk.startswith(f"step{k}/state{i}/block")}
+                assert blocks == {bk for bk in opt.state[p] if bk != 0}
+                for bk in blocks:
+                    st = opt.state[p][bk]
+                    for km in ("scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2"):
+                        ref = d[f"step{k}/state{i}/block{bk}/{km}"]
+                        assert tuple(st[km].shape) == tuple(ref.shape) and st[km].dtype == ref.dtype
+                        fix = torch.abs if km.endswith("exp_avg_2") else (lambda t: t)  # the refreshed basis is free in its signs
+                        assert torch.allclose(fix(st[km].cpu()), fix(ref), rtol=2e-3, atol=1e-6 * max(1.0, ref.abs().max().item())), (k, i, bk, km)
+                    for li in range(3):
+                        gk = f"step{k}/state{i}/block{bk}/scale_by_soap_GG_3/{li}"
+                        if gk in d:
+                            assert torch.allclose(st["scale_by_soap_GG_3"][li].cpu(), d[gk], rtol=1e-4, atol=1e-8)
                 ok = f"step{k}/state{i}/mars_mars_old_grad_5"
                 if ok in d:  # MARS keeps the raw gradient of the step before: a copy
                     assert torch.equal(opt.state[p][0]["mars_mars_old_grad_5"].cpu(), d[ok])
@@ -461,10 +478,10 @@ def test_soap_narrow_storage_matches_oracle(kwargs, rounding):
                 assert torch.equal(opt.state[p][0][km], opt2.state[p2][0][km])
 
 
-@pytest.mark.parametrize("seed", range(20))
+@pytest.mark.parametrize("seed", range(28))
 def test_random_soap_configurations_match_oracle(seed):
     """Seeded draws over SOAP's switches (MARS, caution, decay, max_precond_dim down to sizes that drop a side, precondition_1d,
-    palm, merge_dims, the four clip kinds on the gradient and on the update) and shapes (matrices of aspect ratio at most 2, so that both
+    palm, merge_dims, split, the four clip kinds on the gradient and on the update) and shapes (matrices of aspect ratio at most 2, so that both
     factors have full rank by the first refresh and the refreshed basis is determined by the data; vectors; a stack that
     is merged), seven steps with two refreshes, the step to 5e-3 against the oracle."""
     import random
@@ -491,8 +508,62 @@ def test_random_soap_configurations_match_oracle(seed):
         kwargs.update(palm=True, beta2_scale=rnd.choice([0.6, 0.8]))
     if rnd.random() < 0.3:
         kwargs["merge_dims"] = False
+    per_tensor = ("l2_clip_", "rmsnorm_clip_")
+    if (rnd.random() < 0.35 and not (kwargs["mars"] or kwargs["caution"] or kwargs["precondition_1d"] or kwargs.get("merge_dims") is False)
+            and kwargs.get("gradient_clipping") not in per_tensor and kwargs.get("update_clipping") not in per_tensor):  # fmt: skip
+        # split: blocks of at most 16 x 16 with remainders of 8, so that every block's factors have full rank by the first refresh
+        kwargs.update(split=True, max_precond_dim=16)
+        dims = [16, 24, 32, 40, 48]
+        shapes = [(rnd.choice(dims), rnd.choice(dims)) for _ in range(rnd.randint(1, 3))] + [(rnd.choice([5, 16, 40]),), (2, 3, 40)]
     print("case", seed, kwargs, shapes, flush=True)
     _run_soap_vs_oracle(shapes, kwargs, 7, 5e-3)
+
+
+def test_soap_split_checkpoint_round_trip_and_refusals():
+    """split=True: a checkpoint carries one state per block (``state[p][k]``), and a second optimizer loaded from it continues
+    bit for bit.  State outside the preconditioner, narrow storage and per-block norms are refused at construction."""
+    shapes = [(40, 24), (16,), (2, 3, 40)]
+    host, params = H.make_params(shapes, DEV, scale=0.5)
+    kwargs = dict(split=True, max_precond_dim=16, precondition_frequency=3)
+    opt = heavyball_amd.SOAP(params, **kwargs)
+    for k in range(1, 5):
+        for p, g in zip(params, H.make_grads(shapes, k, torch.float32, 1e-2)):
+            p.grad = g.to(DEV)
+        opt.step()
+    assert sorted(k for k in opt.state[params[0]] if isinstance(k, int)) == [0, 1, 2, 3, 4, 5]  # 3 x 2 blocks of (40, 24)
+    assert tuple(opt.state[params[0]][2]["scale_by_soap_exp_avg_2"].shape) == (1, 8, 16)
+    assert sorted(k for k in opt.state[params[2]] if isinstance(k, int)) == [0, 1, 2]  # (2, 120) in blocks of 16 columns ... merged first
+    params2 = [torch.nn.Parameter(p.detach().clone()) for p in params]
+    opt2 = heavyball_amd.SOAP(params2, **kwargs)
+    opt2.load_state_dict(opt.state_dict())  # straight from the live optimizer: the loaded state must not share memory with it
+    for k in range(5, 7):
+        grads = H.make_grads(shapes, k, torch.float32, 1e-2)
+        for o, ps in ((opt, params), (opt2, params2)):
+            for p, g in zip(ps, grads):
+                p.grad = g.to(DEV)
+            o.step()
+    torch.cuda.synchronize()
+    for p, p2 in zip(params, params2):
+        assert torch.equal(p.detach(), p2.detach())
+    buf = io.BytesIO()  # and through a file, read back with weights_only
+    torch.save(opt.state_dict(), buf)
+    buf.seek(0)
+    opt2.load_state_dict(torch.load(buf, weights_only=True))
+    for k in range(7, 9):
+        grads = H.make_grads(shapes, k, torch.float32, 1e-2)
+        for o, ps in ((opt, params), (opt2, params2)):
+            for p, g in zip(ps, grads):
+                p.grad = g.to(DEV)
+            o.step()
+    torch.cuda.synchronize()
+    for p, p2 in zip(params, params2):
+        assert torch.equal(p.detach(), p2.detach())
+        for bk in opt.state[p]:
+            assert torch.equal(opt.state[p][bk]["scale_by_soap_exp_avg_2"], opt2.state[p2][bk]["scale_by_soap_exp_avg_2"])
+    for bad in (dict(mars=True), dict(caution=True), dict(ecc="bf16+8"), dict(param_ecc="bf16+8"), dict(storage_dtype="bfloat16"),
+                dict(gradient_clipping="l2_clip_"), dict(update_clipping="rmsnorm_clip_")):  # fmt: skip
+        with pytest.raises(NotImplementedError):
+            heavyball_amd.SOAP([torch.nn.Parameter(torch.zeros(4, 4, device=DEV))], split=True, **bad)
 
 
 def test_soap_and_muon_step_over_empty_scalar_and_degenerate_tensors():

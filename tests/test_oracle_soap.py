@@ -87,5 +87,19 @@ def test_soap_trajectory_matches_reference(path):
                 assert (gg is None) == (gk not in d)
                 if gg is not None:
                     assert torch.allclose(gg, d[gk], rtol=1e-4, atol=1e-8)
+            # a split parameter: the further blocks, in the reference's order, each with its own moments and factors
+            blocks = {int(kk.split("/")[2][5:]) for kk in d if kk.startswith(f"step{k}/state{i}/block")}
+            assert blocks == set(orc.block_state[i])
+            for bk in blocks:
+                st = orc.block_state[i][bk]
+                for key in (orc.K_M, orc.K_V):
+                    ref = d[f"step{k}/state{i}/block{bk}/{key}"]
+                    assert tuple(st[key].shape) == tuple(ref.shape)
+                    assert torch.allclose(st[key], ref, rtol=1e-3, atol=1e-6), (k, i, bk, key)
+                for li, gg in enumerate(st[orc.K_GG]):
+                    gk = f"step{k}/state{i}/block{bk}/{orc.K_GG}/{li}"
+                    assert (gg is None) == (gk not in d)
+                    if gg is not None:
+                        assert torch.allclose(gg, d[gk], rtol=1e-4, atol=1e-8)
     if "c5" in path:
         assert [s + 1 for s, f in enumerate(orc.fired) if f] == [11]
