@@ -159,6 +159,135 @@ __device__ __forceinline__ void wait_vmcnt(int n) {  // s_waitcnt vmcnt(n) only 
   }
 }
 
+// The epilogue of both product kernels.  Accumulator register r of tile (i, j) of a wavefront holds row
+// (r/4)*8 + (lane/32)*4 + r%4, column lane%32 of the 32 x 32 block.
+//
+// The row-major bf16 outputs go through LDS: in its registers a lane holds one column of a block, so straight from them a
+// row-major store is two bytes wide (256 to 512 store instructions per lane and tile, which kept the texture-address
+// unit busy for a tenth of a 4096^3 product).  Instead a wavefront writes the 32 rows of a band (its WTN columns) into a
+// region of its own, row after row with 16 bytes of padding (so that the rows of lanes 32..63, four further down, fall
+// on other banks), and reads them back as 16-byte runs of a row, which leave as 16-byte stores.  `lds` is that region
+// (kEpiBytes<WTN> bytes per wavefront); the caller has put a barrier between the main loop's last fragment read and this.
+template <int WTN>
+constexpr int kEpiRow = WTN * 2 + 16;  // bytes per staged row
+template <int WTN>
+constexpr int kEpiBytes = 2 * 32 * kEpiRow<WTN>;  // two outputs (S and Y of the first product)
+
+template <int MODE, int TM, int TN, int WTM, int WTN>
+__device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Problem& g, const int round_out, const int row0, const int col0,
+                                            const int wm, const int wn, const int lane, const int bi, const int bj, char* lds) {
+  constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
+  constexpr bool kRowMajor16 = MODE == kModeS || MODE == kModeY2 || MODE == kModeX;  // a bf16 row-major output exists
+  constexpr int LROW = kEpiRow<WTN>;
+  const int erow = (lane >> 5) * 4, lcol = lane & 31;
+  // the staged band back out: 32 rows x WTN columns in 16-byte runs, 64 of them per pass
+  auto flush_band = [&](const char* region, uint16_t* base, int ld, int row_tile) {
+    constexpr int RUNS = WTN / 8;  // per row
+#pragma unroll
+    for (int t = 0; t < 32 * RUNS / 64; ++t) {
+      const int idx = t * 64 + lane, r = idx / RUNS, ch = idx % RUNS;
+      const uint4 v = *reinterpret_cast<const uint4*>(region + r * LROW + ch * 16);
+      *reinterpret_cast<uint4*>(base + (size_t)(row_tile + r) * ld + col0 + wn * WTN + ch * 8) = v;
+    }
+  };
+  // Transposed copies (X^T, the mirror of a symmetric tile).  A lane holds 4 + 4 + 4 + 4 rows of one column, lane + 32 the
+  // rows between them; v_permlane32_swap trades halves so that a lane below 32 ends up with rows 0..15 of its column and
+  // its partner with rows 16..31, 32 contiguous bytes of the transposed matrix each (64 per column) instead of 8.
+  auto store_transposed = [&](uint16_t* base, int ld, int col, int row_tile, const uint32_t (&v)[16]) {
+    uint32_t pk[4][2], out[8];
+#pragma unroll
+    for (int rb4 = 0; rb4 < 4; ++rb4) {
+      pk[rb4][0] = v[rb4 * 4 + 0] | (v[rb4 * 4 + 1] << 16);
+      pk[rb4][1] = v[rb4 * 4 + 2] | (v[rb4 * 4 + 3] << 16);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)  // h = 0: rows 0-7 | 16-23, h = 1: rows 8-15 | 24-31
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(pk[h][w], pk[h + 2][w], false, false);
+        out[h * 4 + w] = sw[0];      // rows +0..3 of the octet
+        out[h * 4 + 2 + w] = sw[1];  // rows +4..7
+      }
+    uint4* dst = reinterpret_cast<uint4*>(base + (size_t)col * ld + row_tile + (lane >> 5) * 16);
+    dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
+    dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
+  };
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = col0 + wn * WTN + j * 32 + lcol;
+      const int row_tile = row0 + wm * WTM + i * 32;
+      uint32_t prim[16], sec[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int row = row_tile + (q >> 2) * 8 + erow + (q & 3);
+        uint32_t h = f32_to_bf16_rne(acc[i][j][q]);
+        if (MODE == kModeS) {
+          uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * g.mul_c);       // heavyball/utils.py:569
+          if (row == col) y = f32_to_bf16_rne(bf16_to_f32(y) + g.diag);  // :570
+          sec[q] = y;
+        } else if (MODE == kModeY2) {
+          if (row == col) h = f32_to_bf16_rne(bf16_to_f32(h) + g.diag);  // :572
+        }
+        prim[q] = h;
+      }
+#pragma unroll
+      for (int rb4 = 0; rb4 < 4; ++rb4) {
+        const int row = row_tile + rb4 * 8 + erow;
+        if (MODE == kModeFinal || MODE == kModePartial) {
+          float o[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            if (MODE == kModePartial) {
+              o[r] = acc[i][j][rb4 * 4 + r];  // one K chunk of a split product: summed and rounded by ns_split_reduce_kernel
+            } else {
+              o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
+              if (round_out) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
+            }
+          }
+          if (g.f_transposed) {
+            // the 4 consecutive rows of X are 16 contiguous bytes of the output's row `col`
+            float* dst = g.F + (size_t)col * g.ldf + row;
+            if (col < g.f_rows && row + 3 < g.f_cols && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+              *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                if (col < g.f_rows && row + r < g.f_cols) dst[r] = o[r];
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (row + r < g.f_rows && col < g.f_cols) g.F[(size_t)(row + r) * g.ldf + col] = o[r];
+          }
+        } else {
+          uint16_t* stage = reinterpret_cast<uint16_t*>(lds + (rb4 * 8 + erow) * LROW) + j * 32 + lcol;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) stage[r * (LROW / 2)] = (uint16_t)prim[rb4 * 4 + r];
+          if (MODE == kModeS) {
+            stage += 32 * LROW / 2;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) stage[r * (LROW / 2)] = (uint16_t)sec[rb4 * 4 + r];
+          }
+        }
+      }
+      if constexpr (MODE == kModeX) store_transposed(g.C2, g.ldc2, col, row_tile, prim);  // X^T, the B operand of the next iteration
+      // Symmetric modes: a tile above the diagonal is also written transposed to its place below it.  Diagonal tiles
+      // are computed in full, so a matrix that fits one tile gets the plain product.
+      if (SYMMETRIC && bi != bj) {
+        store_transposed(g.C, g.ldc, col, row_tile, prim);
+        if constexpr (MODE == kModeS) store_transposed(g.C2, g.ldc2, col, row_tile, sec);
+      }
+    }
+    if constexpr (kRowMajor16) {
+      const int row_tile = row0 + wm * WTM + i * 32;
+      flush_band(lds, g.C, g.ldc, row_tile);
+      if constexpr (MODE == kModeS) flush_band(lds + 32 * LROW, g.C2, g.ldc2, row_tile);
+    }
+  }
+}
+
 template <int BM, int BN, int BK, int STAGES, int WGM, int WGN, int MODE>
 __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs grp) {
   constexpr int NW = WGM * WGN;
@@ -272,97 +401,208 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
     }
   }
 
-  // epilogue: accumulator register r of tile (i, j) holds row (r/4)*8 + (lane/32)*4 + r%4, column lane%32
-  const int erow = (lane >> 5) * 4, lcol = lane & 31;
-  // Transposed copies (X^T, the mirror of a symmetric tile).  A lane holds 4 + 4 + 4 + 4 rows of one column, lane + 32 the
-  // rows between them; v_permlane32_swap trades halves so that a lane below 32 ends up with rows 0..15 of its column and
-  // its partner with rows 16..31, 32 contiguous bytes of the transposed matrix each (64 per column) instead of 8.
-  auto store_transposed = [&](uint16_t* base, int ld, int col, int row_tile, const uint32_t (&v)[16]) {
-    uint32_t pk[4][2], out[8];
+  static_assert(NW * kEpiBytes<WTN> <= STAGES * STAGE, "the epilogue stages its rows in the ring");
+  __syncthreads();  // nobody reads fragments any more
+  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj, smem + wave * kEpiBytes<WTN>);
+}
+
+// The 256 x 256 tile class: four wavefronts of 128 x 128 (one per SIMD, accumulators in the accumulation registers),
+// K-tiles of 32 in a ring of four.  A wavefront per SIMD has nobody to hide its waits behind, so the instruction stream
+// is laid out by hand: every fragment read and every direct-to-LDS load is issued in the shadow of one matrix
+// instruction (a 32 x 32 x 16 MFMA occupies the pipe for eight issue slots of the wavefront; at most three other
+// instructions follow each one here), and the steady-state loop carries no conditions: the first and the last tiles run
+// a conditional copy of the same body.  Per tile and compute unit this moves 64 KB of fragments out of LDS and 32 KB
+// into it, against 256 KB + 64 KB per 64 of K for eight wavefronts of 128 x 64, which kept LDS busier than the matrix
+// pipes.  One barrier per tile, in its middle: past it, tile kt + 1 has landed for everyone and nobody reads tile kt any more
+// (the fragments of its second k-step are in registers), so its slot is refilled while that k-step is multiplied.
+// The order of the additions into an accumulator is that of ns_gemm_kernel: the two kernels return the same bits.
+template <int V>
+using ns_ic = std::integral_constant<int, V>;
+
+template <int OFF>
+__device__ __forceinline__ bf16x8 lds_read_b128_off(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "16-bit offset field");
+  bf16x8 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+  return v;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void ns_gemm4_kernel(const GroupArgs grp) {
+  constexpr int BM = 256, BN = 256, BK = 32, STAGES = 4, WGN = 2;
+  constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
+  constexpr int ROWB = BK * 2;                  // bytes per LDS row
+  constexpr int STAGE = (BM + BN) * ROWB;       // 32 KB: A's 256 rows, then B's
+  constexpr int LOADS = 8;                      // direct-to-LDS loads (16 rows each) per wavefront and K-tile: 128 rows of one operand
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
+  int pi, bi, bj;
+  const group_ptr_t ka = (group_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+  if (!locate_tile<SYMMETRIC>(ka, blockIdx.x, pi, bi, bj)) return;
+  Problem g;
+  g.A = ka->p[pi].A; g.B = ka->p[pi].B; g.C = ka->p[pi].C; g.C2 = ka->p[pi].C2; g.F = ka->p[pi].F;
+  g.K = ka->p[pi].K; g.lda = ka->p[pi].lda; g.ldb = ka->p[pi].ldb; g.ldc = ka->p[pi].ldc; g.ldc2 = ka->p[pi].ldc2; g.ldf = ka->p[pi].ldf;
+  g.f_rows = ka->p[pi].f_rows; g.f_cols = ka->p[pi].f_cols; g.f_transposed = ka->p[pi].f_transposed; g.scale = ka->p[pi].scale;
+  g.mul_c = ka->p[pi].mul_c; g.diag = ka->p[pi].diag;
+  const int row0 = bi * BM, col0 = bj * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int KT = g.K / BK;
+
+  // Loads: wavefronts 0 and 1 bring A's rows 0..127 and 128..255, wavefronts 2 and 3 B's.  One instruction moves 16 rows
+  // of 64 B: lane l lands in row l / 4, slot l % 4 and fetches the k-chunk that the swizzle keeps in that slot.  The source
+  // is a wavefront-uniform base (operand, first row, K-tile) plus a 32-bit lane offset.
+  const int half = wave & 1;
+  const int ld = wave < 2 ? g.lda : g.ldb;
+  const char* base = wave < 2 ? reinterpret_cast<const char*>(g.A + (size_t)(row0 + half * 128) * g.lda)
+                              : reinterpret_cast<const char*>(g.B + (size_t)(col0 + half * 128) * g.ldb);
+  const int lrow = lane >> 2, lslot = lane & 3;
+  uint32_t voff[LOADS];
 #pragma unroll
-    for (int rb4 = 0; rb4 < 4; ++rb4) {
-      pk[rb4][0] = v[rb4 * 4 + 0] | (v[rb4 * 4 + 1] << 16);
-      pk[rb4][1] = v[rb4 * 4 + 2] | (v[rb4 * 4 + 3] << 16);
-    }
-#pragma unroll
-    for (int h = 0; h < 2; ++h)  // h = 0: rows 0-7 | 16-23, h = 1: rows 8-15 | 24-31
-#pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        const auto sw = __builtin_amdgcn_permlane32_swap(pk[h][w], pk[h + 2][w], false, false);
-        out[h * 4 + w] = sw[0];      // rows +0..3 of the octet
-        out[h * 4 + 2 + w] = sw[1];  // rows +4..7
-      }
-    uint4* dst = reinterpret_cast<uint4*>(base + (size_t)col * ld + row_tile + (lane >> 5) * 16);
-    dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
-    dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
-  };
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = col0 + wn * WTN + j * 32 + lcol;
-      const int row_tile = row0 + wm * WTM + i * 32;
-      uint32_t prim[16], sec[16];
-#pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        const int row = row_tile + (q >> 2) * 8 + erow + (q & 3);
-        uint32_t h = f32_to_bf16_rne(acc[i][j][q]);
-        if (MODE == kModeS) {
-          uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * g.mul_c);       // heavyball/utils.py:569
-          if (row == col) y = f32_to_bf16_rne(bf16_to_f32(y) + g.diag);  // :570
-          sec[q] = y;
-        } else if (MODE == kModeY2) {
-          if (row == col) h = f32_to_bf16_rne(bf16_to_f32(h) + g.diag);  // :572
-        }
-        prim[q] = h;
-      }
-#pragma unroll
-      for (int rb4 = 0; rb4 < 4; ++rb4) {
-        const int row = row_tile + rb4 * 8 + erow;
-        if (MODE == kModeFinal || MODE == kModePartial) {
-          float o[4];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            if (MODE == kModePartial) {
-              o[r] = acc[i][j][rb4 * 4 + r];  // one K chunk of a split product: summed and rounded by ns_split_reduce_kernel
-            } else {
-              o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
-              if (grp.round_out) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
-            }
-          }
-          if (g.f_transposed) {
-            // the 4 consecutive rows of X are 16 contiguous bytes of the output's row `col`
-            float* dst = g.F + (size_t)col * g.ldf + row;
-            if (col < g.f_rows && row + 3 < g.f_cols && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
-              *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-            } else {
-#pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (col < g.f_rows && row + r < g.f_cols) dst[r] = o[r];
-            }
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (row + r < g.f_rows && col < g.f_cols) g.F[(size_t)(row + r) * g.ldf + col] = o[r];
-          }
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) g.C[(size_t)(row + r) * g.ldc + col] = (uint16_t)prim[rb4 * 4 + r];
-          if (MODE == kModeS) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) g.C2[(size_t)(row + r) * g.ldc2 + col] = (uint16_t)sec[rb4 * 4 + r];
-          }
-        }
-      }
-      if constexpr (MODE == kModeX) store_transposed(g.C2, g.ldc2, col, row_tile, prim);  // X^T, the B operand of the next iteration
-      // Symmetric modes: a tile above the diagonal is also written transposed to its place below it.  Diagonal tiles
-      // are computed in full, so a matrix that fits one tile gets the plain product.
-      if (SYMMETRIC && bi != bj) {
-        store_transposed(g.C, g.ldc, col, row_tile, prim);
-        if constexpr (MODE == kModeS) store_transposed(g.C2, g.ldc2, col, row_tile, sec);
-      }
-    }
+  for (int i = 0; i < LOADS; ++i) {
+    const int r = i * 16 + lrow;  // row inside the wavefront's 128 (a multiple of 128 further in the tile: the swizzle does not see it)
+    voff[i] = (uint32_t)(r * ld * 2 + ((lslot ^ ((r >> 2) & 3)) << 4));
   }
+  auto issue_one = [&](int kt, auto i_c) {
+    constexpr int i = decltype(i_c)::value;
+    char* dst = smem + (kt % STAGES) * STAGE + (wave * LOADS + i) * 1024;
+    const char* src = base + (size_t)kt * (BK * 2);
+    __builtin_amdgcn_global_load_lds((gptr_t)(src + voff[i]), (lptr_t)dst, 16, 0, 0);
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // Fragment addresses: row i * 32 + frag_row of the wavefront's 128, chunk ks * 2 + frag_k, swizzled by (row / 4) & 3, which
+  // depends on the lane alone; k-step 1 sits at the address of k-step 0 with bit 5 flipped.  Slots 2 and 3 lie beyond the
+  // 16-bit offset field, so they get base registers of their own.
+  const int frag_row = lane & 31, frag_k = lane >> 5;
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lptr_t)smem;
+  const uint32_t swz = (uint32_t)((frag_k ^ ((frag_row >> 2) & 3)) << 4);
+  uint32_t fa[2][2], fb[2][2];  // [k-step][slot / 2]
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      fa[ks][h] = smem_base + h * 2 * STAGE + (wm * WTM + frag_row) * ROWB + (swz ^ (ks << 5));
+      fb[ks][h] = smem_base + h * 2 * STAGE + (BM + wn * WTN + frag_row) * ROWB + (swz ^ (ks << 5));
+    }
+  bf16x8 afr[2][TM], bfr[2][TN];
+  // fragment r (0..3: A's, 4..7: B's) of k-step ks of the tile in slot sl, into set
+  auto read_one = [&](auto sl_c, auto ks_c, auto set_c, auto r_c) {
+    constexpr int sl = decltype(sl_c)::value, ks = decltype(ks_c)::value, set = decltype(set_c)::value, r = decltype(r_c)::value;
+    constexpr int off = (sl & 1) * STAGE + (r & 3) * 32 * ROWB;
+    if constexpr (r < 4) afr[set][r] = lds_read_b128_off<off>(fa[ks][sl >> 1]);
+    else bfr[set][r - 4] = lds_read_b128_off<off>(fb[ks][sl >> 1]);
+  };
+  // the 16 MFMAs of one k-step on fragment set `cur`; extra(m) is issued right behind MFMA m
+  auto mfmas = [&](auto cur_c, auto&& extra) {
+    constexpr int cur = decltype(cur_c)::value;
+    auto one = [&](auto m_c) {
+      constexpr int m = decltype(m_c)::value, i = m / TN, j = m % TN;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[cur][i], bfr[cur][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      extra(m_c);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // nothing moves across this point: the compiler does not know that the wait in front of the k-step is what makes the
+    // fragments (read through inline assembly) valid, and would hoist the first MFMA above it
+    __builtin_amdgcn_sched_barrier(0);
+    one(ns_ic<0>{}); one(ns_ic<1>{}); one(ns_ic<2>{}); one(ns_ic<3>{}); one(ns_ic<4>{}); one(ns_ic<5>{}); one(ns_ic<6>{}); one(ns_ic<7>{});
+    one(ns_ic<8>{}); one(ns_ic<9>{}); one(ns_ic<10>{}); one(ns_ic<11>{}); one(ns_ic<12>{}); one(ns_ic<13>{}); one(ns_ic<14>{}); one(ns_ic<15>{});
+  };
+  // Tile kt, in slot kt % STAGES, its first fragments already in set 0.  STEADY: tiles kt + 1 and kt + STAGES exist, and
+  // kt >= 1; otherwise the same body with its conditions.
+  auto tile = [&](int kt, auto slot_c, auto steady_c) {
+    constexpr int slot = decltype(slot_c)::value;
+    constexpr bool STEADY = decltype(steady_c)::value;
+    constexpr int nslot = (slot + 1) % STAGES;
+    // k-step 0: behind the first eight MFMAs the fragments of k-step 1 (they then have the other eight to arrive in), behind
+    // four of the rest the second half of the refill that the tile before began (into the slot that tile left at its barrier)
+    wait_lgkmcnt<0>();
+    const bool refill0 = kt >= 1 && kt - 1 + STAGES < KT;
+    mfmas(ns_ic<0>{}, [&](auto m_c) {
+      constexpr int m = decltype(m_c)::value;
+      if constexpr (m < 8) read_one(slot_c, ns_ic<1>{}, ns_ic<1>{}, ns_ic<m>{});
+      else if constexpr (m % 2 == 1) {
+        if (STEADY || refill0) issue_one(kt - 1 + STAGES, ns_ic<4 + (m - 8) / 2>{});
+      }
+    });
+    wait_lgkmcnt<0>();  // every read of tile kt is done
+    const bool more = kt + 1 < KT;
+    if (STEADY || more) {
+      // tile kt + 1 must have landed.  Issued so far: the tiles up to kt - 1 + STAGES; still allowed in flight: those
+      // younger than kt + 1 (loads complete in order)
+      if constexpr (STEADY) {
+        wait_vmcnt((STAGES - 2) * LOADS);
+      } else {
+        const int last_issued = KT - 1 < kt - 1 + STAGES ? KT - 1 : kt - 1 + STAGES;
+        const int younger = last_issued - (kt + 1);
+        if (younger <= 0) wait_vmcnt(0);
+        else if (younger == 1) wait_vmcnt(LOADS);
+        else if (younger == 2) wait_vmcnt(2 * LOADS);
+        else wait_vmcnt(0);
+      }
+      __builtin_amdgcn_s_barrier();
+    }
+    // k-step 1: behind the first eight MFMAs the first fragments of tile kt + 1, behind four of the rest the first half of
+    // the refill of this tile's slot with tile kt + STAGES
+    const bool refill = kt + STAGES < KT;
+    mfmas(ns_ic<1>{}, [&](auto m_c) {
+      constexpr int m = decltype(m_c)::value;
+      if constexpr (m < 8) {
+        if (STEADY || more) read_one(ns_ic<nslot>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<m>{});
+      } else if constexpr (m % 2 == 1) {
+        if (STEADY || refill) issue_one(kt + STAGES, ns_ic<(m - 8) / 2>{});
+      }
+    });
+  };
+  // prologue: the ring is filled, tile 0 has landed for everyone, its first fragments are on their way
+  for (int s = 0; s < STAGES && s < KT; ++s) {
+    issue_one(s, ns_ic<0>{}); issue_one(s, ns_ic<1>{}); issue_one(s, ns_ic<2>{}); issue_one(s, ns_ic<3>{});
+    issue_one(s, ns_ic<4>{}); issue_one(s, ns_ic<5>{}); issue_one(s, ns_ic<6>{}); issue_one(s, ns_ic<7>{});
+  }
+  {
+    const int younger = (KT < STAGES ? KT : STAGES) - 1;
+    if (younger <= 0) wait_vmcnt(0);
+    else if (younger == 1) wait_vmcnt(LOADS);
+    else if (younger == 2) wait_vmcnt(2 * LOADS);
+    else wait_vmcnt(3 * LOADS);
+  }
+  __builtin_amdgcn_s_barrier();
+  read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}); read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<1>{});
+  read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<2>{}); read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<3>{});
+  read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<4>{}); read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<5>{});
+  read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<6>{}); read_one(ns_ic<0>{}, ns_ic<0>{}, ns_ic<0>{}, ns_ic<7>{});
+  // the first group conditionally (tile 0 has no refill half behind it), the steady groups while the last tile of a group
+  // still has its tile kt + STAGES, the rest conditionally again
+  int kt = 0;
+  tile(0, ns_ic<0>{}, std::false_type{});
+  if (1 < KT) tile(1, ns_ic<1>{}, std::false_type{});
+  if (2 < KT) tile(2, ns_ic<2>{}, std::false_type{});
+  if (3 < KT) tile(3, ns_ic<3>{}, std::false_type{});
+  for (kt = STAGES; kt + 2 * STAGES - 1 < KT; kt += STAGES) {
+    tile(kt, ns_ic<0>{}, std::true_type{});
+    tile(kt + 1, ns_ic<1>{}, std::true_type{});
+    tile(kt + 2, ns_ic<2>{}, std::true_type{});
+    tile(kt + 3, ns_ic<3>{}, std::true_type{});
+  }
+  for (; kt < KT; kt += STAGES) {
+    tile(kt, ns_ic<0>{}, std::false_type{});
+    if (kt + 1 < KT) tile(kt + 1, ns_ic<1>{}, std::false_type{});
+    if (kt + 2 < KT) tile(kt + 2, ns_ic<2>{}, std::false_type{});
+    if (kt + 3 < KT) tile(kt + 3, ns_ic<3>{}, std::false_type{});
+  }
+
+  static_assert(4 * kEpiBytes<WTN> <= STAGES * STAGE, "the epilogue stages its rows in the ring");
+  __syncthreads();  // nobody reads fragments any more
+  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj, smem + wave * kEpiBytes<WTN>);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -627,14 +867,22 @@ static int launch_group(const GroupArgs& a, int n_blocks, hipStream_t s) {
   return HB_OK;
 }
 
+template <int MODE>
+static int launch_group4(const GroupArgs& a, int n_blocks, hipStream_t s) {
+  constexpr int smem = 4 * (256 + 256) * 32 * 2;
+  static LdsReservation reserved;
+  auto kern = ns_gemm4_kernel<MODE>;
+  const void* kp = reinterpret_cast<const void*>(kern);
+  if (int rc = reserve_lds(reserved, &kp, 1, smem, "hb_ns5")) return rc;
+  kern<<<n_blocks, 256, smem, s>>>(a);
+  return HB_OK;
+}
+
 // One product of the iteration for every matrix of one tile class: matrices are listed longest K first (the hardware
 // starts workgroups in id order, so the long tiles start first and the short ones fill in behind them) and launched
 // in groups of at most kMaxGroup.
 template <int MODE>
 static int gemm_stage(std::vector<Problem> probs, int tile, hipStream_t s, int round_out = 0) {
-#ifndef HB_GEMM_CFG
-#define HB_GEMM_CFG 256, 256, 64, 2, 4, 2
-#endif
   constexpr bool symmetric = MODE == kModeS || MODE == kModeY2;
   std::stable_sort(probs.begin(), probs.end(), [](const Problem& a, const Problem& b) { return a.K > b.K; });
   for (size_t first = 0; first < probs.size(); first += kMaxGroup) {
@@ -652,7 +900,7 @@ static int gemm_stage(std::vector<Problem> probs, int tile, hipStream_t s, int r
 #ifndef HB_GEMM_CFG_SMALL
 #define HB_GEMM_CFG_SMALL 128, 128, 64, 2, 2, 4
 #endif
-    const int rc = tile == 256 ? launch_group<HB_GEMM_CFG, MODE>(a, blocks, s) : launch_group<HB_GEMM_CFG_SMALL, MODE>(a, blocks, s);
+    const int rc = tile == 256 ? launch_group4<MODE>(a, blocks, s) : launch_group<HB_GEMM_CFG_SMALL, MODE>(a, blocks, s);
     if (rc) return rc;
   }
   return HB_OK;
