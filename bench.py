@@ -301,7 +301,7 @@ def bench_muon(steps=5, warmup=2):
             "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "traffic": None,
             "algorithmic_flops_per_step": flops,
-            "kernel": "hb::ns_gemm_kernel (15 grouped launches over all matrices inside hb_ns5_batched, plus norm and conversion kernels)",
+            "kernel": "hb::ns_gemm4_kernel (15 grouped launches over all matrices inside hb_ns5_batched, plus norm and conversion kernels)",
         },
     }
 

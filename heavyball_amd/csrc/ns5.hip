@@ -161,35 +161,11 @@ __device__ __forceinline__ void wait_vmcnt(int n) {  // s_waitcnt vmcnt(n) only 
 
 // The epilogue of both product kernels.  Accumulator register r of tile (i, j) of a wavefront holds row
 // (r/4)*8 + (lane/32)*4 + r%4, column lane%32 of the 32 x 32 block.
-//
-// The row-major bf16 outputs go through LDS: in its registers a lane holds one column of a block, so straight from them a
-// row-major store is two bytes wide (256 to 512 store instructions per lane and tile, which kept the texture-address
-// unit busy for a tenth of a 4096^3 product).  Instead a wavefront writes the 32 rows of a band (its WTN columns) into a
-// region of its own, row after row with 16 bytes of padding (so that the rows of lanes 32..63, four further down, fall
-// on other banks), and reads them back as 16-byte runs of a row, which leave as 16-byte stores.  `lds` is that region
-// (kEpiBytes<WTN> bytes per wavefront); the caller has put a barrier between the main loop's last fragment read and this.
-template <int WTN>
-constexpr int kEpiRow = WTN * 2 + 16;  // bytes per staged row
-template <int WTN>
-constexpr int kEpiBytes = 2 * 32 * kEpiRow<WTN>;  // two outputs (S and Y of the first product)
-
 template <int MODE, int TM, int TN, int WTM, int WTN>
 __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Problem& g, const int round_out, const int row0, const int col0,
-                                            const int wm, const int wn, const int lane, const int bi, const int bj, char* lds) {
+                                            const int wm, const int wn, const int lane, const int bi, const int bj) {
   constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
-  constexpr bool kRowMajor16 = MODE == kModeS || MODE == kModeY2 || MODE == kModeX;  // a bf16 row-major output exists
-  constexpr int LROW = kEpiRow<WTN>;
   const int erow = (lane >> 5) * 4, lcol = lane & 31;
-  // the staged band back out: 32 rows x WTN columns in 16-byte runs, 64 of them per pass
-  auto flush_band = [&](const char* region, uint16_t* base, int ld, int row_tile) {
-    constexpr int RUNS = WTN / 8;  // per row
-#pragma unroll
-    for (int t = 0; t < 32 * RUNS / 64; ++t) {
-      const int idx = t * 64 + lane, r = idx / RUNS, ch = idx % RUNS;
-      const uint4 v = *reinterpret_cast<const uint4*>(region + r * LROW + ch * 16);
-      *reinterpret_cast<uint4*>(base + (size_t)(row_tile + r) * ld + col0 + wn * WTN + ch * 8) = v;
-    }
-  };
   // Transposed copies (X^T, the mirror of a symmetric tile).  A lane holds 4 + 4 + 4 + 4 rows of one column, lane + 32 the
   // rows between them; v_permlane32_swap trades halves so that a lane below 32 ends up with rows 0..15 of its column and
   // its partner with rows 16..31, 32 contiguous bytes of the transposed matrix each (64 per column) instead of 8.
@@ -262,13 +238,11 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
               if (row + r < g.f_rows && col < g.f_cols) g.F[(size_t)(row + r) * g.ldf + col] = o[r];
           }
         } else {
-          uint16_t* stage = reinterpret_cast<uint16_t*>(lds + (rb4 * 8 + erow) * LROW) + j * 32 + lcol;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) stage[r * (LROW / 2)] = (uint16_t)prim[rb4 * 4 + r];
+          for (int r = 0; r < 4; ++r) g.C[(size_t)(row + r) * g.ldc + col] = (uint16_t)prim[rb4 * 4 + r];
           if (MODE == kModeS) {
-            stage += 32 * LROW / 2;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) stage[r * (LROW / 2)] = (uint16_t)sec[rb4 * 4 + r];
+            for (int r = 0; r < 4; ++r) g.C2[(size_t)(row + r) * g.ldc2 + col] = (uint16_t)sec[rb4 * 4 + r];
           }
         }
       }
@@ -279,11 +253,6 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
         store_transposed(g.C, g.ldc, col, row_tile, prim);
         if constexpr (MODE == kModeS) store_transposed(g.C2, g.ldc2, col, row_tile, sec);
       }
-    }
-    if constexpr (kRowMajor16) {
-      const int row_tile = row0 + wm * WTM + i * 32;
-      flush_band(lds, g.C, g.ldc, row_tile);
-      if constexpr (MODE == kModeS) flush_band(lds + 32 * LROW, g.C2, g.ldc2, row_tile);
     }
   }
 }
@@ -401,9 +370,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
     }
   }
 
-  static_assert(NW * kEpiBytes<WTN> <= STAGES * STAGE, "the epilogue stages its rows in the ring");
-  __syncthreads();  // nobody reads fragments any more
-  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj, smem + wave * kEpiBytes<WTN>);
+  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj);
 }
 
 // The 256 x 256 tile class: four wavefronts of 128 x 128 (one per SIMD, accumulators in the accumulation registers),
@@ -600,9 +567,7 @@ __global__ __launch_bounds__(256) void ns_gemm4_kernel(const GroupArgs grp) {
     if (kt + 3 < KT) tile(kt + 3, ns_ic<3>{}, std::false_type{});
   }
 
-  static_assert(4 * kEpiBytes<WTN> <= STAGES * STAGE, "the epilogue stages its rows in the ring");
-  __syncthreads();  // nobody reads fragments any more
-  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj, smem + wave * kEpiBytes<WTN>);
+  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
