@@ -346,7 +346,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
   // per K-tile: once through it, tile kt is in LDS for everyone and everyone has finished reading tile kt-1, whose slot
   // then takes tile kt+STAGES-1.  Inside a tile the fragments of k-step s+1 are fetched while step s is multiplied.
   // With eight wavefronts per workgroup (two per SIMD) the hardware interleaves one wavefront's waits with the other's
-  // matrix instructions; that measured faster than four wavefronts with a hand-interleaved instruction stream.
+  // matrix instructions.  This kernel serves the 128 x 128 tile class; the 256 x 256 class runs on ns_gemm4_kernel below.
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
     if (s < KT) issue_loads(s);
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
 // instruction (a 32 x 32 x 16 MFMA occupies the pipe for eight issue slots of the wavefront; at most three other
 // instructions follow each one here), and the steady-state loop carries no conditions: the first and the last tiles run
 // a conditional copy of the same body.  Per tile and compute unit this moves 64 KB of fragments out of LDS and 32 KB
-// into it, against 256 KB + 64 KB per 64 of K for eight wavefronts of 128 x 64, which kept LDS busier than the matrix
+// into it, against 256 KB + 64 KB per 64 of K for eight wavefronts of 64 x 128, which kept LDS busier than the matrix
 // pipes.  One barrier per tile, in its middle: past it, tile kt + 1 has landed for everyone and nobody reads tile kt any more
 // (the fragments of its second k-step are in registers), so its slot is refilled while that k-step is multiplied.
 // The order of the additions into an accumulator is that of ns_gemm_kernel: the two kernels return the same bits.
