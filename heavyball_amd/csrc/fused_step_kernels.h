@@ -153,25 +153,31 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
     if constexpr (kLazy) {
       bool need = false;
       uint32_t fast = 0;
+      // Bounds, all on the safe side.  A bf16 + int8 pair lies within 2^(max(e, 1) - 135) of its primary x (e its exponent
+      // field), which is at most max(|x| 2^-8, 2^-126) <= |x| 2^-8 + 2^-126: with x times a coefficient already at hand
+      // (t2, s1) the bound costs one multiply.  The factors 1.01 cover the roundings of the bound arithmetic itself.
+      const float k_ulp = 1.01f * 0x1p-8f;
+      const float c_o = __builtin_fabsf(a.amars) * (1.01f * 0x1p-126f);
+      const float c_m = __builtin_fabsf(a.oma1) * (1.01f * 0x1p-126f);
+      const float k_a1 = __builtin_fabsf(a.a1) * 1.01f;
 #pragma unroll
       for (int j = 0; j < kE; ++j) {
         const uint32_t hm = (rm[k].a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
         const float mp = bf16_to_f32(hm);
-        const float half_ulp_m = ldexpf(1.0f, ecc_log_scale<true>(hm));  // bound on |decoded - primary|
         float gs = g[j], dg = 0.0f;
         bool sure = true;
         if (MARS) {
           const uint32_t ho = (ro[k].a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
           const float t1 = g[j] * a.omamars, t2 = bf16_to_f32(ho) * a.amars;
           gs = t1 + t2;  // the corrected gradient before its rounding, from the primary of old_grad
-          const float eo = __builtin_fabsf(a.amars) * ldexpf(1.0f, ecc_log_scale<true>(ho)) * 1.01f +
-                           (__builtin_fabsf(t1) + __builtin_fabsf(t2)) * 0x1p-22f;  // what the correction and fp32 rounding can move
+          // what the correction of old_grad and the fp32 roundings can move
+          const float eo = __builtin_fabsf(t2) * k_ulp + (__builtin_fabsf(t1) + __builtin_fabsf(t2)) * 0x1p-22f + c_o;
           sure = __builtin_fabsf(gs) > eo;  // its sign is settled (the stochastic rounding to bf16 keeps the sign)
           dg = eo + (__builtin_fabsf(gs) + eo) * 0x1p-7f + 1e-39f;  // ... and its value to within one bf16 ulp more
         }
         const float s1 = mp * a.oma1, s2 = gs * a.a1;
         const float mn = s1 + s2;
-        const float em = (__builtin_fabsf(a.oma1) * half_ulp_m + __builtin_fabsf(a.a1) * dg) * 1.01f + (__builtin_fabsf(s1) + __builtin_fabsf(s2)) * 0x1p-21f;
+        const float em = __builtin_fabsf(s1) * k_ulp + k_a1 * dg + (__builtin_fabsf(s1) + __builtin_fabsf(s2)) * 0x1p-21f + c_m;
         sure = sure && __builtin_fabsf(mn) > em;  // NaN compares false: the exact route decides
         const bool inside = FULL || e + j < valid;
         need = need || (inside && !sure);
