@@ -306,6 +306,43 @@ def bench_muon(steps=5, warmup=2):
     }
 
 
+def bench_muonadamw_gpt2(steps=10, warmup=3):
+    """MuonAdamW (heavyball/__init__.py:475-540) on the headline parameter set: the 49 matrices of the GPT-2-small-shaped set go
+    through Muon (momentum, Newton-Schulz on the 128 x 128 tile class, the embedding's first product split along K), the 98
+    vectors through Adam; one optimizer, one step counter."""
+    import torch
+
+    import heavyball_amd
+
+    dev = torch.device("cuda:0")
+    shapes = gpt2_small_shapes()
+    torch.manual_seed(2)
+    params = [torch.nn.Parameter(torch.randn(s, device=dev) * 0.02) for s in shapes]
+    opt = heavyball_amd.MuonAdamW(params)
+    grads = [torch.randn(s, device=dev) * 1e-2 for s in shapes]
+
+    def one_step():
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.step()
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    flops = sum(ns5_flops(*s) for s in shapes if len(s) == 2)
+    return {
+        "workload": "MuonAdamW defaults, GPT-2-small-shaped 147 tensors (49 matrices through Newton-Schulz, 98 vectors through Adam), fp32",
+        "ms_per_step": round(ms_step, 3),
+        "ns5_algorithmic_flops_per_step": flops,
+        "tflops_if_all_of_the_step_were_newton_schulz": round(flops / (ms_step * 1e-3) / 1e12, 1),
+    }
+
+
 def bench_reference_script(steps=300, warmup=20, windows=6):
     """The reference's own micro-benchmark (benchmarks/bench_optimizer_step.py:13, :53-81): AdamW with default arguments and
     consume_grad=False on 32 fp32 tensors of [2048, 2048] (134,217,728 elements), 20 warm-up steps, then 6 windows of 300
@@ -567,6 +604,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_muon:
         out["ns5"] = bench_muon()
+        out["muonadamw_gpt2"] = bench_muonadamw_gpt2()
     if not args.no_soap:
         torch.cuda.empty_cache()
         out["soap"] = bench_soap()
