@@ -19,7 +19,7 @@ ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD, FLAG_MARS_ONLY = 1, 2, 4, 8, 16, 32, 64, 128
 RNG_HALF, RNG_PHILOX = 0, 1
 STREAM_MARS_SR, STREAM_PARAM, STREAM_EXP_AVG, STREAM_EXP_AVG_SQ, STREAM_OLD_GRAD, STREAM_INIT_PARAM, STREAM_NS_INPUT = range(7)
-STREAM_CLIP, STREAM_EXP_AVG_SLOW, STREAM_UPDATE, STREAM_SOAP_ROTATE = 8, 9, 10, 11
+STREAM_CLIP, STREAM_EXP_AVG_SLOW, STREAM_UPDATE, STREAM_SOAP_ROTATE, STREAM_UPDATE_CLIP = 8, 9, 10, 11, 12
 NS_LEGACY, NS_BF16_UPDATE = 1, 2
 NOALLOC_MAX_TENSORS = 65536  # HB_NOALLOC_MAX_TENSORS
 GEMM_ACCUMULATE, GEMM_SYMMETRIC = 1, 2

@@ -117,6 +117,25 @@ def debiased_weights(beta: torch.Tensor, step) -> Tuple[float, float]:
         return float(a), float(one - a)
 
 
+_ONE32 = np.float32(1)
+
+
+def debiased_weights_np(beta: float, n: int) -> Tuple[float, float]:
+    """``debiased_weights`` for a python-float beta and a python-int step, on numpy scalars throughout.  The power of a 0-d fp32
+    tensor by a 0-d int64 tensor is the C library's ``powf`` on the CPU, and so is numpy's ``float32 ** float32``
+    (tests/test_host_logic.py compares the two over many steps), which makes the whole chain a handful of 0.1-microsecond operations."""
+    b = np.float32(beta)
+    with np.errstate(all="ignore"):
+        a = _ONE32 - (_ONE32 - (_ONE32 - b) / (_ONE32 - b ** np.float32(n)))
+        return float(a), float(_ONE32 - a)
+
+
+def step_lr_np(base_lr: float, n: int, warmup_steps: int) -> np.float32:
+    """``base_lr * step / step.clamp(min=warmup_steps + 1)`` of heavyball/chainable.py:2560 with ``step`` an int64 0-d tensor: the
+    python float is rounded to fp32, the product and the quotient are single fp32 operations."""
+    return np.float32(base_lr) * np.float32(n) / np.float32(max(n, warmup_steps + 1))
+
+
 def current_stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -218,6 +237,7 @@ class HBOptimizer(torch.optim.Optimizer):
         base.setdefault("multi_tensor", True)
         self._buckets: Dict[int, List[Bucket]] = {}
         self._loc: Dict[int, Tuple[Bucket, int]] = {}  # id(parameter) -> (bucket, index in the bucket)
+        self._plans: Dict[int, "_StepPlan"] = {}  # group index -> cached launch plan of the fused step (FirstOrder._fast_step)
         self.rng_seed = int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF
         self.use_ema = False
         self.inner_group = {}
@@ -250,6 +270,8 @@ class HBOptimizer(torch.optim.Optimizer):
 
     def add_param_group(self, param_group):
         super().add_param_group(param_group)
+        if hasattr(self, "_plans"):
+            self._plans.clear()
         if hasattr(self, "_buckets"):
             gi = len(self.param_groups) - 1
             if gi not in self._buckets and getattr(self, "_constructed", False):
@@ -394,10 +416,13 @@ class HBOptimizer(torch.optim.Optimizer):
                 self._step(gi, group)
         return loss
 
-    def _step(self, gi: int, group: dict):
-        """heavyball/chainable.py:2510-2570."""
-        if gi not in self._buckets:
-            self._adopt_group(gi, group)
+    def _fast_step(self, gi: int, group: dict) -> bool:
+        """A step from a cached launch plan; False when there is none or it does not fit this step (the general path runs then)."""
+        return False
+
+    @staticmethod
+    def _note_lr(group: dict):
+        """heavyball/chainable.py:2542-2551: the learning rate the group is stepped with is remembered; a change is reported once."""
         if "base_lr" not in group:
             group["base_lr"] = group["lr"]
         elif group["base_lr"] != group["lr"]:
@@ -406,6 +431,14 @@ class HBOptimizer(torch.optim.Optimizer):
                 f"only supported with multi_tensor=True (currently multi_tensor={group['multi_tensor']})."
             )
             group["base_lr"] = group["lr"]
+
+    def _step(self, gi: int, group: dict):
+        """heavyball/chainable.py:2510-2570."""
+        if gi in self._plans and self._fast_step(gi, group):
+            return
+        if gi not in self._buckets:
+            self._adopt_group(gi, group)
+        self._note_lr(group)
         caution = group["caution"]
         active = []
         for p in group["params"]:
@@ -572,6 +605,7 @@ class HBOptimizer(torch.optim.Optimizer):
                 v = dict(v)  # not the caller's object: two optimizers loaded from one checkpoint must not share a counter
             setattr(self, k, v)
         sd = {k: v for k, v in state_dict.items() if k != "heavyball"}
+        self._plans.clear()
         super().load_state_dict(sd)
         self._rehome_state()
 
@@ -619,6 +653,18 @@ class HBOptimizer(torch.optim.Optimizer):
 # ---------------------------------------------------------------------------------------------------------------
 # AdamW / LaProp on the fused kernel
 # ---------------------------------------------------------------------------------------------------------------
+class _BucketPlan:
+    """What one bucket's launch needs from step to step: the filled descriptor and the tables it points to."""
+
+    __slots__ = ("bucket", "desc", "gdt", "params", "home", "keep", "device_index")
+
+
+class _StepPlan:
+    """The launches of one parameter group as the general path last issued them, for ``FirstOrder._fast_step``."""
+
+    __slots__ = ("sig", "buckets", "step_t", "state0", "n_state", "lr_t", "mars_key", "mars_w")
+
+
 class FirstOrder(HBOptimizer):
     """AdamW-, LaProp-, ADOPT-, AdEMAMix- and NAdam-style optimizers: one call of ``hb_fused_step`` per parameter bucket."""
 
@@ -661,9 +707,18 @@ class FirstOrder(HBOptimizer):
         names = list(self._moment_keys(group).values()) + ([k_o] if mars else [])
         ready = b.state_ready.setdefault((tuple(names), prim, corr), set())
         if len(ready) == len(b.params) or ready.issuperset(idx):
-            if names[0] in self.state[b.params[idx[0]]].get(0, ()):
+            # the caller may have dropped entries of optimizer.state since (all of them, or one parameter's): look at every one
+            state, params, first = self.state, b.params, names[0]
+            for i in idx:
+                st = state.get(params[i])
+                if st is None or first not in st.get(0, ()):
+                    stale = set(ready)  # tensors whose slab ranges still hold the moments of the dropped entries
+                    ready.clear()  # build the entries again
+                    break
+            else:
                 return
-            ready.clear()  # optimizer.state was emptied by the caller: build the entries again
+        else:
+            stale = ()
         for k in names:
             b.slab.role(k, prim)
             if corr is not None:
@@ -674,9 +729,14 @@ class FirstOrder(HBOptimizer):
             if names[0] in st and (not mars or k_o in st):
                 continue
             for k in names:
+                fresh = k not in st
                 st.setdefault(k, b.slab.view(k, i))
                 if corr is not None:
                     st.setdefault(k + "::ecc", b.slab.view(k + "::ecc", i))
+                if fresh and i in stale:  # a dropped entry starts from zero again, as the reference's zero_guard would
+                    st[k].zero_()
+                    if corr is not None:
+                        st[k + "::ecc"].zero_()
             st.setdefault("is_initialized", set()).update(init_ids)
         ready.update(idx)
 
@@ -699,6 +759,88 @@ class FirstOrder(HBOptimizer):
     def _fill_bucket(self, d, b: Bucket, lst, group, step):
         """Per-bucket descriptor fields beyond the common ones; returns what must stay alive until the stream is done."""
         return None
+
+    #: the step's scalars and descriptor are those of this class (no per-step hooks of a subclass): ``_fast_step`` may replay them
+    _plannable = False
+
+    def _plan_signature(self, group) -> tuple:
+        """Everything, apart from the hyper-parameters that ``_fast_step`` reads afresh, that decides how a step is launched."""
+        return (group["caution"], bool(group.get("mars", False)), bool(group.get("cautious_weight_decay", False)), group.get("ecc"),
+                group.get("param_ecc"), group.get("storage_dtype"), self.rounding, self.promote, self.mars_write_grad,
+                self.gradient_clipping, self.update_clipping, self._use_palm)  # fmt: skip
+
+    def _fast_step(self, gi: int, group: dict) -> bool:
+        """The step of a group whose every parameter has a gradient of the dtype, alignment and layout of the step before: the
+        descriptors of that step are launched again with the new step number, scalars and gradient pointers.  Nothing is
+        computed differently from the general path (tests/test_host_logic.py compares the scalars, the GPU tests the steps);
+        anything out of the ordinary - a missing or differently typed gradient, a parameter whose data was rebound, emptied
+        optimizer state, changed switches - returns False before anything was touched, and the general path takes the step."""
+        plan = self._plans[gi]
+        step_t = plan.step_t
+        if (plan.sig != self._plan_signature(group) or group.get("_group_step") is not step_t or plan.state0.get("step") is not step_t
+                or len(self.state) != plan.n_state):  # fmt: skip
+            del self._plans[gi]
+            return False
+        base_lr = group["lr"]
+        if type(base_lr) is not float:
+            return False
+        self._note_lr(group)
+        staged = []
+        for bp in plan.buckets:
+            grads = [p.grad for p in bp.params]
+            try:
+                ptrs = [g.data_ptr() for g in grads]
+            except (AttributeError, RuntimeError):  # a parameter without a gradient, or a gradient without dense storage
+                return False
+            gdt = bp.gdt
+            for g in grads:
+                if g.dtype is not gdt or not g.is_contiguous():
+                    return False
+            low = 0
+            for a in ptrs:
+                low |= a
+            if low & 15 or [p.data_ptr() for p in bp.params] != bp.home:
+                return False
+            staged.append(ptrs)
+        if self.consume_grad:
+            for bp in plan.buckets:
+                for p in bp.params:
+                    p.grad = None
+        n = step_t.item() + 1
+        step_t.fill_(n)
+        lr = step_lr_np(base_lr, n, group["warmup_steps"])
+        group["prev_lr"] = plan.lr_t.fill_(float(lr))
+        betas = group["betas"]
+        beta1 = betas[0] if group.get("beta") is None else group["beta"]
+        a1, oma1 = debiased_weights_np(beta1, n)
+        a2, oma2 = debiased_weights_np(betas[1], n)
+        eps = float(np.float32(group["eps"] if self._algo == _lib.ALGO_ADAM else 1e-8))
+        omdl, neg_lr = float(_ONE32 - np.float32(group["weight_decay"]) * lr), float(-lr)
+        if plan.sig[1]:
+            key = (group["mars_gamma"], beta1)
+            if plan.mars_key != key:
+                plan.mars_key, plan.mars_w = key, mars_weights(group)
+            mars_a, mars_oma = plan.mars_w
+        else:
+            mars_a, mars_oma = 0.0, 1.0
+        L = _lib.lib()
+        seed, step32 = self.rng_seed, n & 0xFFFFFFFF
+        current = torch.cuda.current_device()
+        for bp, ptrs in zip(plan.buckets, staged):
+            b, d = bp.bucket, bp.desc
+            table = b.grad_ptr_table(bp.gdt, ptrs)
+            d.grad_ptrs = table.data_ptr()
+            d.a1, d.one_minus_a1, d.a2, d.one_minus_a2, d.eps = a1, oma1, a2, oma2, eps
+            d.mars_a, d.one_minus_mars_a, d.neg_lr, d.one_minus_decay_lr = mars_a, mars_oma, neg_lr, omdl
+            d.step, d.seed = step32, seed
+            if bp.device_index == current:
+                rc = L.hb_fused_step(d, current_stream_ptr(b.device))
+            else:
+                with torch.cuda.device(b.device):
+                    rc = L.hb_fused_step(d, current_stream_ptr(b.device))
+            _lib.check(rc, "hb_fused_step")
+            self._last_launch = (d, (table, bp.keep))
+        return True
 
     #: take the un-fused form of the transform (scale_by_*, then update_param_) whenever a gradient is narrower than fp32: the
     #: reference's un-fused transform leaves its result in an update buffer of the gradient's dtype (MuonAdamW's vector route)
@@ -744,6 +886,7 @@ class FirstOrder(HBOptimizer):
             per_bucket.setdefault(id(b), [b, []])[1].append((i, p, g))
 
         work = []  # (bucket, [(index, gradient)], gradient dtype)
+        as_given = True  # every gradient went to the kernel as the caller handed it over (no cast, no copy)
         for b, items in per_bucket.values():
             if b.device.type != "cuda":
                 raise _lib.HbError("the optimizer step runs on the GPU only: parameters must live on a CUDA/HIP device")
@@ -756,11 +899,11 @@ class FirstOrder(HBOptimizer):
                     raise NotImplementedError("sparse gradients")
                 dt = g.dtype
                 if dt is not f32_t and (promote or dt not in _PLAIN_FMT):
-                    g, dt = g.float(), f32_t
+                    g, dt, as_given = g.float(), f32_t, False
                 if g.shape != p.shape:
                     raise ValueError(f"gradient shape {tuple(g.shape)} does not match parameter shape {tuple(p.shape)}")
                 if g.data_ptr() & 15 or not g.is_contiguous() or g.device != b.device:
-                    g = g.detach().to(b.device).clone(memory_format=torch.contiguous_format)
+                    g, as_given = g.detach().to(b.device).clone(memory_format=torch.contiguous_format), False
                 lst = by_dtype.get(dt)
                 if lst is None:
                     lst = by_dtype[dt] = []
@@ -770,6 +913,7 @@ class FirstOrder(HBOptimizer):
             for gdt, lst in by_dtype.items():
                 lst.sort(key=lambda t: t[0])
                 work.append((b, lst, gdt))
+        prologue = False
         if self.gradient_clipping is not None and mars:
             # heavyball/chainable.py:2694-2699: MARS, then the clip, then the transform.  The prologue runs as a pass of its
             # own (HB_FLAG_MARS_ONLY) that leaves the corrected gradients in the fp32 role "_clip"; the step proper then
@@ -778,11 +922,15 @@ class FirstOrder(HBOptimizer):
                 self._mars_prologue(L, group, b, lst, gdt, step, mars_a, mars_oma, state_fmt, k_o)
             flags &= ~(_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD)
             mars = False
+            prologue = True
             clipped = self._clip_gradients(L, group, work, step, gathered=True)
         elif self.gradient_clipping is not None:
             clipped = self._clip_gradients(L, group, work, step)
         else:
             clipped = [None] * len(work)
+        plannable = (as_given and not unfused and self.gradient_clipping is None and not self._use_palm and self._plannable
+                     and len(active) == len(group["params"]) and len(work) == len(per_bucket))
+        plan_buckets = []
         if not self._begin_step(group, work):  # ADOPT's warm-up: only exp_avg_sq moves (and MARS' old gradient)
             flags = (flags & (_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD)) | _lib.FLAG_ADOPT_WARMUP
             scal = dict(scal, a2=1.0, one_minus_a2=0.0)
@@ -836,18 +984,29 @@ class FirstOrder(HBOptimizer):
                 rc = L.hb_fused_step(d, current_stream_ptr(b.device))
             _lib.check(rc, "hb_fused_step")
             self._last_launch = (d, (table, chunks, offsets, numel, clip, extra))  # kept for profiling harnesses
+            if plannable:
+                bp = _BucketPlan()
+                bp.bucket, bp.desc, bp.gdt, bp.params, bp.home = b, d, gdt, b.params, b.home_ptrs()
+                bp.keep, bp.device_index = (chunks, offsets, numel), b.device.index
+                plan_buckets.append(bp)
+        if plannable:
+            plan = _StepPlan()
+            plan.sig, plan.buckets = self._plan_signature(group), plan_buckets
+            plan.step_t, plan.state0, plan.n_state = group["_group_step"], self._state0(active[0][0]), len(self.state)
+            plan.lr_t, plan.mars_key, plan.mars_w = torch.zeros((), dtype=torch.float32), None, None
+            self._plans[gi] = plan
         if not unfused:
             return
         keep = self._clip_updates(L, [(b, [i for i, _ in lst]) for b, lst, _ in work]) if self.update_clipping is not None else None
         decay_py = group["weight_decay"]  # update_param_ keeps decay a python float (heavyball/utils.py:2393-2406)
-        for b, lst, gdt in work:
+        for (b, lst, gdt), clip in zip(work, clipped):
             upd_role, upd_fmt = "_update", _lib.FMT_F32
             if gdt == torch.bfloat16:
                 # the clip writes its result back into the bf16 update buffer through copy_stochastic_ (heavyball/utils.py:3231)
                 wide, narrow = b.slab.role("_update", torch.float32), b.slab.role("_update16", torch.bfloat16)
                 with torch.cuda.device(b.device):
                     _lib.check(L.hb_sr_bf16(wide.data_ptr(), narrow.data_ptr(), wide.numel(), self._rng_mode(), self.rng_seed,
-                                            int(step) & 0xFFFFFFFF, _lib.STREAM_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
+                                            int(step) & 0xFFFFFFFF, _lib.STREAM_UPDATE_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
                 upd_role, upd_fmt = "_update16", _lib.FMT_BF16
             offsets, numel = b.slab.meta()
             chunks, n_chunks = b.slab.chunks(tuple(i for i, _ in lst))
@@ -858,6 +1017,11 @@ class FirstOrder(HBOptimizer):
             d = _lib.HbStepDesc()
             d.param, d.param_corr = b.slab.ptr("param"), b.slab.ptr("param::ecc")
             d.grad, d.grad_ptrs = None, table.data_ptr()
+            if prologue:
+                # MARS ran as a pass of its own and left the corrected gradients in a slab role instead of the caller's buffers
+                # (heavyball/chainable.py:646 overwrites those); the clip that followed scaled them by a positive factor, which
+                # keeps every sign bit, and the sign is all that caution reads
+                d.grad, d.grad_ptrs, gdt = clip[0].data_ptr(), None, clip[1]
             d.exp_avg, d.state_fmt = b.slab.ptr(upd_role), upd_fmt
             d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
             d.caution_count = b.caution_scratch().data_ptr() if group["caution"] else None
@@ -880,6 +1044,7 @@ class AdamW(FirstOrder):
 
     _algo = _lib.ALGO_ADAM
     _fn_name = "update_by_adam"
+    _plannable = True
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), eps=1e-8, weight_decay=0, cautious_weight_decay: bool = False,
                  warmup_steps=0, multi_tensor: bool = True, storage_dtype: str = "float32", mars: bool = False,
@@ -895,6 +1060,7 @@ class LaProp(FirstOrder):
 
     _algo = _lib.ALGO_LAPROP
     _fn_name = "update_by_laprop"
+    _plannable = True
 
     def __init__(self, params, lr=0.0025, betas=(0.9, 0.99), eps=1e-8, weight_decay=0, cautious_weight_decay: bool = False,
                  warmup_steps=0, multi_tensor: bool = True, storage_dtype: str = "float32", mars: bool = False,

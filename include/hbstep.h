@@ -103,6 +103,8 @@ enum {
   HB_STREAM_EXP_AVG_SLOW = 9, /* AdEMAMix's slow momentum */
   HB_STREAM_UPDATE = 10,      /* HB_FLAG_UPDATE_ONLY with bf16 gradients: the update is rounded to bf16 as the reference's update buffer is */
   HB_STREAM_SOAP_ROTATE = 11, /* SOAP: exp_avg written back to bf16 / ECC storage after its rotation into a refreshed basis */
+  HB_STREAM_UPDATE_CLIP = 12, /* bf16 stochastic rounding of a clipped bf16 update (update_clipping with bf16 gradients); its own
+                                 stream, so that a step with both clips draws independent noise for the two roundings */
 };
 
 /*

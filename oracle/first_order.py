@@ -513,7 +513,7 @@ class FirstOrderOracle:
                 fn = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip,
                       "global_rmsnorm_clip": global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
                 for u, c, t in zip(update, fn(update), idx):
-                    copy_stochastic(u, c, rounding, philox.STREAM_CLIP, t)
+                    copy_stochastic(u, c, rounding, philox.STREAM_UPDATE_CLIP, t)
             # the tail of the chain decays with the group's weight_decay whatever the transform did with it (NAdam: on top of its own)
             update_param_(p, update, lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)
             return

@@ -43,6 +43,7 @@ STREAM_CLIP = 8  # bf16 stochastic rounding of a clipped bf16 gradient
 STREAM_EXP_AVG_SLOW = 9  # ECC / SR write of AdEMAMix's slow momentum
 STREAM_UPDATE = 10  # rounding of an un-fused transform's update into a 16-bit update buffer (update clipping)
 STREAM_SOAP_ROTATE = 11  # ECC / SR write of SOAP's exp_avg after its rotation into a refreshed eigenbasis
+STREAM_UPDATE_CLIP = 12  # bf16 stochastic rounding of a clipped bf16 update (independent of STREAM_CLIP, the gradient clip's)
 
 
 def philox4x32_10(c0, c1, c2, c3, k0, k1):

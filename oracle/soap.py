@@ -145,7 +145,12 @@ def adam_(exp_avg, exp_avg_sq, grad: Tensor, beta1, beta2, step: Tensor, eps, ro
 
 def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg, rounding=None, tidx=0):
     """heavyball/utils.py:829-900 (heavy=False): one power-iteration step + QR per side, then rotate exp_avg into the new basis
-    (decoded to fp32 for the rotation and written back through copy_stochastic_, :883-884)."""
+    (decoded to fp32 for the rotation and written back through copy_stochastic_, :883-884).
+
+    Returns the smallest gap between two neighbouring sort keys (the estimates ``diag(Q^T GG Q)`` that order the columns, :871-873)
+    relative to the largest one, over all sides; 1.0 when nothing was sorted.  The order of two keys that agree to fp32 rounding
+    is decided by the summation order of the products, so a checker can tell from this figure when the column order - and with it
+    the rotated exp_avg - is not determined by the data."""
     from . import first_order as fo
     from . import philox
     from .rounding import HalfRounding
@@ -153,14 +158,18 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
     stored = exp_avg
     exp_avg = fo.promote(stored)
     if exp_avg.dim() <= 1:
-        return
+        return 1.0
     new_qs = []
+    key_gap = 1.0
     for m, q in zip(GG, Q):
         if m is None:
             new_qs.append(None)
             continue
         tmp = m @ q
         eig = torch.einsum("...ij,...ij->...j", q, tmp)
+        if eig.shape[-1] > 1:
+            keys = eig.double().sort(dim=-1, descending=True).values
+            key_gap = min(key_gap, ((keys[..., :-1] - keys[..., 1:]).min() / keys.abs().max().clamp_min(1e-300)).item())
         idx = torch.argsort(eig, descending=True).unsqueeze(-2).expand_as(tmp)
         tmp.scatter_(-1, idx, torch.linalg.qr(tmp.gather(-1, idx)).Q)
         new_qs.append(tmp)
@@ -168,7 +177,7 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
     in_str, out_str = einsum_base[:pd], einsum_base[pd : 2 * pd]
     from_sh = ",".join([f"...{o}{i}" for m, i, o in zip(Q, in_str, in_str.upper()) if m is not None])
     if not from_sh:
-        return
+        return key_gap
     to_sh = ",".join([f"...{i}{o}" for m, i, o in zip(new_qs, in_str.upper(), out_str) if m is not None])
     out_lin = "".join([o if o in to_sh else i for i, o in zip(in_str, out_str)])
     subs = f"...{in_str},{from_sh},{to_sh}->...{out_lin}"
@@ -177,6 +186,7 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
     for q, qn in zip(Q, new_qs):
         if q is not None:
             q.copy_(qn)
+    return key_gap
 
 
 class SOAPOracle:
@@ -226,6 +236,7 @@ class SOAPOracle:
         self.state = self._state_init
         self.step_count = torch.zeros((), dtype=torch.int64)
         self.fired = []
+        self.sort_key_gap = {}  # (tensor, block) -> smallest relative gap of the sort keys over the refreshes so far
 
     def _moment(self, st, key, like):
         """zero_guard with the group's storage (heavyball/chainable.py:277-301)."""
@@ -301,7 +312,8 @@ class SOAPOracle:
                 beta = beta_debias(self.shampoo_beta, step)  # heavyball/chainable.py:1244
                 update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta)
                 if is_precond:
-                    refresh_basis(GG, Q, m_st, rounding, i)
+                    gap = refresh_basis(GG, Q, m_st, rounding, i)
+                    self.sort_key_gap[(i, k)] = min(self.sort_key_gap.get((i, k), 1.0), gap)
                 todo_p.append(p)
                 todo_u.append(precond.squeeze(0).reshape(p.shape))
                 todo_g.append(g)

@@ -318,6 +318,19 @@ def make_clip_combinations():
                                                                          caution=True), shapes, torch.float32, 4)  # fmt: skip
 
 
+def make_both_clips():
+    """MARS, a gradient clip, an update clip and caution in one chain (heavyball/chainable.py:2693-2701): caution's sign test in the
+    chain's tail reads the gradient as MARS left it (heavyball/chainable.py:646), not the raw one."""
+    shapes = [(4, 8), (16,), (3, 5)]
+    run_traj("adamw_mars_clip_updclip_caution", heavyball.AdamW, dict(mars=True, gradient_clipping="l2_clip_", update_clipping="rmsnorm_clip_",
+                                                                      caution=True, weight_decay=0.01, mars_gamma=0.5), shapes, torch.float32, 5,
+             grad_scale=1.0)  # fmt: skip
+    run_traj("laprop_mars_clip_updclip_caution_bf16grad_ecc", heavyball.LaProp, dict(mars=True, gradient_clipping="global_l2norm_clip",
+                                                                                     update_clipping="l2_clip_", caution=True, ecc="bf16+8",
+                                                                                     mars_gamma=0.5, lr=0.01), shapes, torch.bfloat16, 5,
+             grad_scale=1.0)  # fmt: skip
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -475,7 +488,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -490,6 +503,8 @@ if __name__ == "__main__":
         make_palm_trajectories()
     if "clipcombo" in which:
         make_clip_combinations()
+    if "bothclips" in which:
+        make_both_clips()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:

@@ -219,7 +219,7 @@ def _random_case(seed):
     return cls_name, kwargs, gdt, bf16_params, shapes, none_for, rnd.choice(["half", "philox"])
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(600))
 def test_random_configurations_match_oracle(seed):
     """Seeded draws over optimizer, switches, storage formats, gradient and parameter dtypes and ragged sizes (one element up
     to three chunks, around every multiple of the work unit), three steps each, bit for bit against the oracle: the
@@ -602,3 +602,123 @@ def test_parameter_rebound_after_construction_is_moved_back_into_the_slab():
     params[1].grad = torch.zeros(shapes[1], device=DEV)
     with pytest.raises(_lib.HbError, match="dtype"):
         opt.step()
+
+
+PLAN_CASES = [
+    ("laprop_ecc_bf16grad", heavyball_amd.LaProp, dict(ecc="bf16+8"), torch.bfloat16, 1e-3),
+    ("adamw_mars_caution_ecc_paramecc", heavyball_amd.AdamW, dict(mars=True, caution=True, ecc="bf16+8", param_ecc="bf16+8", weight_decay=0.01),
+     torch.bfloat16, 1e-3),
+    ("adamw_fp32_warmup_decay", heavyball_amd.AdamW, dict(weight_decay=0.1, warmup_steps=3, betas=(0.9, 0.999)), torch.float32, 1e-2),
+]  # fmt: skip
+
+
+@pytest.mark.parametrize("case", PLAN_CASES, ids=[c[0] for c in PLAN_CASES])
+def test_cached_plan_steps_equal_the_general_path(case):
+    """``FirstOrder._fast_step`` replays the launches of the step before with new scalars and gradient pointers.  Two optimizers
+    on the same inputs, one with the cached plan switched off, stay bit-identical through ordinary steps and through everything
+    that must send a step back to the general path: a missing gradient, a changed learning rate and betas (which the plan reads
+    afresh), a gradient of another dtype, a non-contiguous gradient, a parameter rebound to new storage, gradients kept
+    (consume_grad=False), a second param group.  The steps the plan took are counted."""
+    _, cls, kwargs, gdt, gscale = case
+    shapes = [(64, 96), (96,), (1000, 33), (7,)]
+    gen = torch.Generator().manual_seed(0)
+    host = [torch.randn(s, generator=gen) * 0.02 for s in shapes]
+    opts, sets = [], []
+    for planned in (True, False):
+        params = [torch.nn.Parameter(h.clone().to(DEV)) for h in host]
+        for p in params:
+            p.grad_dtype = None
+        opt = cls([dict(params=params[:3]), dict(params=params[3:], lr=1e-3)], **kwargs)
+        opt.rng_seed = 4321
+        if not planned:
+            opt._plannable = False
+        opts.append(opt)
+        sets.append(params)
+    taken = []
+    fast = opts[0]._fast_step
+    opts[0]._fast_step = lambda gi, group: (taken.append(gi) if (ok := fast(gi, group)) else None, ok)[1]
+
+    def grads_for(k, dtype=gdt):
+        g = torch.Generator().manual_seed(1000 + k)
+        return [(torch.randn(s, generator=g) * gscale).to(dtype) for s in shapes]
+
+    def step_both(k, grads):
+        for opt, params in zip(opts, sets):
+            for p, g in zip(params, grads):
+                p.grad = None if g is None else g.to(DEV)
+            opt.step()
+        torch.cuda.synchronize()
+        for i, (p, q) in enumerate(zip(*sets)):
+            H.assert_bit_equal(p.data, q.data, f"step {k} param {i}")
+            sp, sq = opts[0].state[p].get(0, {}), opts[1].state[q].get(0, {})
+            assert set(sp) == set(sq)
+            for key, val in sp.items():
+                if isinstance(val, torch.Tensor):
+                    H.assert_bit_equal(val, sq[key], f"step {k} tensor {i} {key}")
+
+    for k in (1, 2, 3, 4):
+        step_both(k, grads_for(k))
+    # group 1 replays from its second step on; group 0 rebuilds its plan once more when group 1's state entries have appeared
+    assert taken.count(1) == 3 and taken.count(0) >= 2
+    taken.clear()
+    g5 = grads_for(5)
+    g5[1] = None
+    step_both(5, g5)  # a tensor without a gradient: the general path, for group 0 only
+    assert taken == [1]
+    step_both(6, grads_for(6))
+    for opt in opts:
+        opt.param_groups[0]["lr"] = 5e-4
+        opt.param_groups[0]["betas"] = (0.8, 0.95)
+        opt.param_groups[1]["weight_decay"] = 0.05
+    taken.clear()
+    import warnings
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        step_both(7, grads_for(7))
+    assert sorted(taken) == [0, 1]  # new hyper-parameters do not need the general path
+    other = torch.float32 if gdt == torch.bfloat16 else torch.bfloat16
+    taken.clear()
+    step_both(8, grads_for(8, other))  # another gradient dtype: general path, and a new plan from there
+    step_both(9, grads_for(9, other))
+    assert sorted(taken) == [0, 1]
+    step_both(10, grads_for(10))
+    g11 = grads_for(11)
+    g11[0] = g11[0].t().contiguous().t()  # same values, column-major
+    taken.clear()
+    step_both(11, g11)
+    assert taken == [1]
+    for params in sets:
+        params[2].data = params[2].data.clone()  # new storage
+    step_both(12, grads_for(12))
+    step_both(13, grads_for(13))
+    for opt in opts:
+        opt.consume_grad = False
+    taken.clear()
+    step_both(14, grads_for(14))
+    assert sorted(taken) == [0, 1] and all(p.grad is not None for p in sets[0])
+    sd = opts[0].state_dict()
+    opts[0].load_state_dict(sd)  # drops the plans; the tensors of the state move, the values stay
+    taken.clear()
+    step_both(15, grads_for(15))
+    assert taken == []
+    step_both(16, grads_for(16))
+    assert sorted(taken) == [0, 1]
+
+
+def test_dropped_state_entry_starts_from_zero_again():
+    """``del optimizer.state[p]`` for one parameter between steps: its moments restart from zero (the reference's zero_guard
+    builds them anew), the other parameters carry on, and ``state_dict()`` lists the rebuilt entries."""
+    shapes = [(64, 96), (96,), (1000, 33)]
+    host, params, opt, orc = H.build_pair(heavyball_amd.LaProp, "laprop", shapes, dict(ecc="bf16+8"), DEV, rounding="philox")
+    H.run_steps(opt, orc, params, shapes, 3, torch.bfloat16, 1e-3, DEV, tag="before")
+    del opt.state[params[1]]
+    orc.state[1] = {}
+    for k in (4, 5):
+        grads = H.make_grads(shapes, k, torch.bfloat16, 1e-3)
+        for p, g in zip(params, grads):
+            p.grad = g.to(DEV)
+        opt.step()
+        orc.step([g.clone() for g in grads])
+        H.compare(opt, orc, params, f"after the drop, step {k}")
+    assert "update_by_laprop_exp_avg_0" in opt.state_dict()["state"][1][0]

@@ -231,10 +231,22 @@ def _adopt_basis(opt, params, basis_of):
                         q.copy_(basis_of(i, li, k))
 
 
+SORT_KEY_TIE = 1e-5  # relative; fp32 sums of a few thousand products in two orders differ by less
+
+
 def _run_soap_vs_oracle(shapes, kwargs, steps, tol, adopt=True, grad_fn=None, signed=False, diag_tol=1e-4):
+    """Runs the optimizer and the oracle side by side.  Returns (opt, orc, undetermined): a basis refresh orders the new columns by
+    the estimates diag(Q^T GG Q) (heavyball/utils.py:871-873); two estimates that agree to fp32 rounding are ordered by whichever
+    way the products were summed, and the two orders give bases with two columns exchanged while exp_avg_sq stays where it was -
+    both are valid runs of the reference's algorithm and they part from there.  Rule: once the oracle reports two neighbouring
+    sort keys closer than SORT_KEY_TIE of the largest for a tensor, that tensor's rotated exp_avg is not compared at that refresh
+    and the tensor is left out of the later steps (every tensor, if a norm over the whole group enters the update); such tensors
+    are returned in ``undetermined``."""
     host, params = H.make_params(shapes, DEV, scale=0.5)
     opt = heavyball_amd.SOAP(params, **kwargs)
     orc = osoap.SOAPOracle([h.clone() for h in host], **kwargs)
+    undetermined, parted = set(), set()
+    group_norm = kwargs.get("update_clipping") in ("global_l2norm_clip", "global_rmsnorm_clip")
     for k in range(1, steps + 1):
         grads = grad_fn(k) if grad_fn is not None else H.make_grads(shapes, k, torch.float32, 1e-2)
         prev = [p.detach().cpu().clone() for p in params]
@@ -245,7 +257,13 @@ def _run_soap_vs_oracle(shapes, kwargs, steps, tol, adopt=True, grad_fn=None, si
         orc.step([g.clone() for g in grads])
         torch.cuda.synchronize()
         assert bool(opt.param_groups[0]["is_preconditioning"]) == orc.fired[-1]
+        parted |= undetermined  # a tie at an earlier refresh: the two runs have parted since
+        if group_norm and parted:
+            parted = set(range(len(params)))
+        undetermined = {i for (i, _), gap in orc.sort_key_gap.items() if gap < SORT_KEY_TIE}
         for i, p in enumerate(params):
+            if i in parted:
+                continue
             got, want = p.detach().cpu() - prev[i], orc.params[i] - prev_o[i]
             if k == 1:
                 assert torch.equal(p.detach().cpu(), prev[i])  # the first step only initialises
@@ -267,7 +285,10 @@ def _run_soap_vs_oracle(shapes, kwargs, steps, tol, adopt=True, grad_fn=None, si
             # eigenvector signs are free (eigh without an adopted basis; the QR of every refresh): exp_avg in the rotated
             # basis matches up to the sign of each entry
             fix = torch.abs
-            assert rel_fro(fix(st[orc.K_M]), fix(orc.state[i][orc.K_M])) < tol and rel_fro(st[orc.K_V], orc.state[i][orc.K_V]) < tol
+            assert rel_fro(st[orc.K_V], orc.state[i][orc.K_V]) < tol, (k, i)
+            if i in undetermined:
+                continue
+            assert rel_fro(fix(st[orc.K_M]), fix(orc.state[i][orc.K_M])) < tol, (k, i)
             if signed:
                 # with separated eigenvalues the two bases agree column by column up to sign: take the signs from Q and
                 # compare the rotated momentum itself, entry [a, b] carrying sign_left[a] * sign_right[b]
@@ -287,7 +308,7 @@ def _run_soap_vs_oracle(shapes, kwargs, steps, tol, adopt=True, grad_fn=None, si
                     assert rel_fro(st[orc.K_GG][li], gg) < 1e-5
         if k == 1 and adopt:
             _adopt_basis(opt, params, lambda i, li, k: (orc.state[i] if k == 0 else orc.block_state[i][k])[orc.K_Q][li].to(DEV))
-    return opt, orc
+    return opt, orc, undetermined | parted
 
 
 def test_soap_square_factors_own_eigh():
@@ -306,7 +327,7 @@ def test_soap_mid_size_own_eigh_signed_momentum():
     entry by its own magnitude, which carries that angle into the step at full size (measured 4e-4 ... 2e-2; the same
     run at 64 wide agrees to 2e-5)."""
     shapes = [(256, 256), (512, 512)]
-    opt, orc = _run_soap_vs_oracle(shapes, dict(precondition_frequency=3), 7, 3e-2, adopt=False, signed=True)
+    opt, orc, _ = _run_soap_vs_oracle(shapes, dict(precondition_frequency=3), 7, 3e-2, adopt=False, signed=True)
     assert sum(orc.fired) == 2  # the float-accumulated schedule of frequency 3 fires at steps 3 and 7
 
 
@@ -317,7 +338,7 @@ def test_soap_at_benchmark_shapes_matches_oracle():
     refresh (the batched factorisation of four bases at once) and a step in the refreshed basis, the checker's basis adopted
     after the first step, every step to 5e-3.  The checker needs about half a minute of CPU time."""
     shapes = [(2048, 2048), (2048, 8192), (8192, 2048)]
-    opt, orc = _run_soap_vs_oracle(shapes, dict(precondition_frequency=3), 4, 5e-3)
+    opt, orc, _ = _run_soap_vs_oracle(shapes, dict(precondition_frequency=3), 4, 5e-3)
     assert orc.fired == [False, False, True, False]
 
 
@@ -327,7 +348,7 @@ def test_soap_matches_oracle_with_refresh():
     on a rank-deficient factor amplifies rounding differences without bound, on any two implementations.
     Tolerance 2e-3 on the step taken: QR comes from different LAPACK implementations on the two sides."""
     shapes = [(48, 80), (33,), (40, 20), (10, 3, 4)]
-    opt, orc = _run_soap_vs_oracle(shapes, dict(precondition_frequency=4, weight_decay=0.01), 9, 2e-3)
+    opt, orc, _ = _run_soap_vs_oracle(shapes, dict(precondition_frequency=4, weight_decay=0.01), 9, 2e-3)
     assert [s + 1 for s, f in enumerate(orc.fired) if f] == [4, 8]
     sd = opt.state_dict()
     st0 = sd["state"][0][0]
@@ -340,7 +361,7 @@ def test_soap_matches_oracle_with_refresh():
 def test_soap_max_precond_dim_drops_a_side():
     """heavyball/utils.py:1373-1376: a dimension above max_precond_dim gets no factor and no rotation on that side."""
     shapes = [(24, 100), (100, 24)]
-    opt, orc = _run_soap_vs_oracle(shapes, dict(precondition_frequency=4, max_precond_dim=32), 6, 2e-3)
+    opt, orc, _ = _run_soap_vs_oracle(shapes, dict(precondition_frequency=4, max_precond_dim=32), 6, 2e-3)
     p0, p1 = opt.param_groups[0]["params"]
     assert opt.state[p0][0]["scale_by_soap_GG_3"][1] is None and opt.state[p1][0]["scale_by_soap_GG_3"][0] is None
 
@@ -478,7 +499,7 @@ def test_soap_narrow_storage_matches_oracle(kwargs, rounding):
                 assert torch.equal(opt.state[p][0][km], opt2.state[p2][0][km])
 
 
-@pytest.mark.parametrize("seed", range(28))
+@pytest.mark.parametrize("seed", range(200))
 def test_random_soap_configurations_match_oracle(seed):
     """Seeded draws over SOAP's switches (MARS, caution, decay, max_precond_dim down to sizes that drop a side, precondition_1d,
     palm, merge_dims, split, the four clip kinds on the gradient and on the update) and shapes (matrices of aspect ratio at most 2, so that both
@@ -517,6 +538,18 @@ def test_random_soap_configurations_match_oracle(seed):
         shapes = [(rnd.choice(dims), rnd.choice(dims)) for _ in range(rnd.randint(1, 3))] + [(rnd.choice([5, 16, 40]),), (2, 3, 40)]
     print("case", seed, kwargs, shapes, flush=True)
     _run_soap_vs_oracle(shapes, kwargs, 7, 5e-3)
+
+
+def test_soap_configuration_with_tied_sort_keys():
+    """A configuration found by a longer seeded sweep: its [8, 8] tensor reaches the second refresh (step 7) with two sort keys
+    1.4e-7 of the largest apart, one fp32 ulp, so the order of those two columns is a coin toss between summation orders (the
+    CPU suite shows the tie in float64, tests/test_oracle_soap.py).  The comparison must hold on everything the data determines
+    and the rule of _run_soap_vs_oracle must name that tensor, and only that one, as undetermined."""
+    shapes = [(4, 2, 3), (17,), (8, 8), (33, 28)]
+    kwargs = dict(precondition_frequency=3, mars=False, caution=False, weight_decay=0.01, max_precond_dim=2048, precondition_1d=False,
+                  gradient_clipping="global_rmsnorm_clip")  # fmt: skip
+    _, _, undetermined = _run_soap_vs_oracle(shapes, kwargs, 7, 5e-3)
+    assert undetermined == {2}
 
 
 def test_soap_split_checkpoint_round_trip_and_refusals():

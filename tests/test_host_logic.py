@@ -127,6 +127,15 @@ def test_step_scalars_match_reference_bits():
             # the step's own fast path: same bits with the IEEE operations on numpy scalars
             assert optim.debiased_weights(optim.f32(float(b1)), step) == (a1, oma1)
             assert optim.debiased_weights(optim.f32(float(b2)), step) == (a2, oma2)
+            # and the cached-plan step's, which takes the power on numpy scalars too
+            assert optim.debiased_weights_np(float(b1), s) == (a1, oma1)
+            assert optim.debiased_weights_np(float(b2), s) == (a2, oma2)
+    for key, rows in sc.items():
+        if not key.startswith("lr_"):
+            continue
+        _, base_lr, warm = key.split("_")
+        for s, want in enumerate(rows, start=1):
+            assert hx(float(optim.step_lr_np(float(base_lr), s, int(warm)))) == want, (key, s)
 
 
 def test_debiased_weights_equal_the_tensor_pipeline():
@@ -140,6 +149,28 @@ def test_debiased_weights_equal_the_tensor_pipeline():
         for s in steps:
             step = torch.tensor(s, dtype=torch.int64)
             assert optim.debiased_weights(beta, step) == optim.lerp_weights(optim.beta_debias(beta, step)), (b, s)
+            assert optim.debiased_weights_np(b, s) == optim.lerp_weights(optim.beta_debias(beta, step)), (b, s)
+
+
+def test_numpy_step_scalars_equal_the_tensor_pipeline():
+    """The scalars of the cached-plan step (numpy float32 scalars) against the general path's 0-d tensor arithmetic, bit for bit:
+    the learning rate with warm-up, ``1 - decay * lr`` and ``-lr``, over learning rates, warm-ups, decays and steps - including
+    steps beyond 2**24, where the step itself is rounded on its way to fp32."""
+    import numpy as np
+
+    gen = torch.Generator().manual_seed(5)
+    lrs = [1e-3, 0.0025, 3e-3, 1.0, 0.1] + (torch.rand(20, generator=gen) * 1e-2).tolist()
+    steps = list(range(1, 60)) + [1000, 99999, 2**24 + 1, 2**24 + 3, 10**9 + 7]
+    for base_lr in lrs:
+        for warm in (0, 3, 10, 2000):
+            for s in steps:
+                step = torch.tensor(s, dtype=torch.int64)
+                want = optim.f32(base_lr * step / step.clamp(min=warm + 1))
+                got = optim.step_lr_np(base_lr, s, warm)
+                assert float(got) == float(want), (base_lr, warm, s)
+                for decay in (0.0, 0.01, 0.1, 1e-4):
+                    assert float(np.float32(1) - np.float32(decay) * got) == float(1 - optim.f32(decay) * want)
+                assert float(-got) == float(-want)
 
 
 def test_ns_coefficients_follow_cpu_scalar_rounding():

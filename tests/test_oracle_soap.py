@@ -103,3 +103,27 @@ def test_soap_trajectory_matches_reference(path):
                         assert torch.allclose(gg, d[gk], rtol=1e-4, atol=1e-8)
     if "c5" in path:
         assert [s + 1 for s, f in enumerate(orc.fired) if f] == [11]
+
+
+def test_tied_sort_keys_are_reported_and_decide_the_column_order():
+    """A refresh orders the new basis by the estimates diag(Q^T GG Q) (heavyball/utils.py:871-873).  On the configuration below (a
+    seeded draw of the GPU sweep) the [8, 8] tensor reaches its second refresh, at step 7, with two estimates one fp32 ulp apart:
+    the oracle must report that gap, and evaluating the same estimates in float64 must order the two columns the other way or
+    the same way by a margin that fp32 cannot resolve - which is why the GPU comparison leaves such a tensor out from there."""
+    from tests import helpers as H
+
+    shapes = [(4, 2, 3), (17,), (8, 8), (33, 28)]
+    gen = torch.Generator().manual_seed(0)
+    host = [torch.randn(s, generator=gen) * 0.5 for s in shapes]
+    orc = soap.SOAPOracle(host, precondition_frequency=3, weight_decay=0.01, gradient_clipping="global_rmsnorm_clip")
+    for k in range(1, 7):
+        orc.step(H.make_grads(shapes, k, torch.float32, 1e-2))
+    assert all(gap > 1e-4 for gap in orc.sort_key_gap.values())  # the refresh at step 3 is well determined everywhere
+    q_before = orc.state[2][orc.K_Q][0].clone()
+    orc.step(H.make_grads(shapes, 7, torch.float32, 1e-2))
+    assert orc.fired[-1]
+    assert orc.sort_key_gap[(2, 0)] < 1e-6
+    assert min(gap for key, gap in orc.sort_key_gap.items() if key != (2, 0)) > 1e-4
+    gg = orc.state[2][orc.K_GG][0][0].double()
+    keys = ((gg @ q_before[0].double()) * q_before[0].double()).sum(0).sort(descending=True).values
+    assert ((keys[:-1] - keys[1:]).min() / keys[0]).item() < 1e-6  # the tie is in the data, not in the fp32 evaluation
