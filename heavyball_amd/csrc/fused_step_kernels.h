@@ -33,6 +33,9 @@ struct Geo {
 #ifndef HB_GEO_COUNT
 #define HB_GEO_COUNT Geo<8, 2>
 #endif
+#ifndef HB_GEO_F32  // the all-fp32 triple: no codec work at all
+#define HB_GEO_F32 Geo<2, 2>
+#endif
 
 struct StepArgs {
   char* param;
@@ -378,9 +381,8 @@ struct StepKernel {
   int sub;
 };
 
-template <int ALGO, int PF, int GF, int SF>
+template <int ALGO, int PF, int GF, int SF, class S = HB_GEO_STEP>
 inline StepKernel pick_pass(bool mars, int caution) {
-  using S = HB_GEO_STEP;
   using C = HB_GEO_COUNT;
   if (mars) {
     if (caution == kNoCaution) return {fused_step_kernel<ALGO, true, kNoCaution, PF, GF, SF, S>, S::kSub};
@@ -395,9 +397,16 @@ inline StepKernel pick_pass(bool mars, int caution) {
 // The kernel of one algorithm for a (param, grad, state) format triple: three triples are statically specialised,
 // everything else takes the kernel that switches on run-time format codes.  Explicitly instantiated per algorithm in
 // fused_step_algo.hip.
+//
+// The geometry goes with the triple: the less arithmetic a step carries per byte, the less a lane should hold.  Measured on one
+// MI355X (fraction of 8 TB/s, Geo<4,2> / <4,1> / <2,2> / <2,4>): (f32,f32,f32) 0.733 / 0.776 / 0.778 / 0.763, (f32,bf16,f32)
+// 0.766 / 0.803 / 0.808 / 0.772, (bf16,bf16,f32) 0.775 / 0.806 / 0.767 / 0.792, (f32,f32,bf16) 0.760 / 0.787 / 0.738 / 0.799,
+// (f32,f32,ecc) 0.757 / 0.773 / 0.711 / 0.754, while the triples with the most arithmetic, (f32,bf16,ecc) 0.767 / 0.735 / 0.689 /
+// 0.722, (ecc,bf16,ecc) with MARS 0.722 / 0.712 / 0.636 / 0.629 and (bf16,bf16,bf16) 0.679 / 0.611 / 0.510 / 0.561, want Geo<4,2>.
 template <int ALGO>
 StepKernel pick_algo(bool mars, int caution, int pf, int gf, int sf) {
-  if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_F32) return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_F32>(mars, caution);
+  if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_F32)
+    return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_F32, HB_GEO_F32>(mars, caution);
   if (pf == HB_FMT_F32 && gf == HB_FMT_BF16 && sf == HB_FMT_ECC_BF16_8)
     return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_ECC_BF16_8>(mars, caution);
   if (pf == HB_FMT_ECC_BF16_8 && gf == HB_FMT_BF16 && sf == HB_FMT_ECC_BF16_8)
@@ -405,12 +414,16 @@ StepKernel pick_algo(bool mars, int caution, int pf, int gf, int sf) {
   // mixed-precision set-ups without ECC, for the two optimizers they are mostly run with: bf16 parameters and gradients over
   // fp32 or bf16 moments, fp32 parameters with bf16 gradients (measured 4.6 / 3.3 / 5.2 TB/s on the run-time-format kernel)
   if constexpr (ALGO == HB_ALGO_ADAM || ALGO == HB_ALGO_LAPROP) {
-    if (pf == HB_FMT_BF16 && gf == HB_FMT_BF16 && sf == HB_FMT_F32) return pick_pass<ALGO, HB_FMT_BF16, HB_FMT_BF16, HB_FMT_F32>(mars, caution);
+    if (pf == HB_FMT_BF16 && gf == HB_FMT_BF16 && sf == HB_FMT_F32)
+      return pick_pass<ALGO, HB_FMT_BF16, HB_FMT_BF16, HB_FMT_F32, Geo<4, 1>>(mars, caution);
     if (pf == HB_FMT_BF16 && gf == HB_FMT_BF16 && sf == HB_FMT_BF16) return pick_pass<ALGO, HB_FMT_BF16, HB_FMT_BF16, HB_FMT_BF16>(mars, caution);
-    if (pf == HB_FMT_F32 && gf == HB_FMT_BF16 && sf == HB_FMT_F32) return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_F32>(mars, caution);
+    if (pf == HB_FMT_F32 && gf == HB_FMT_BF16 && sf == HB_FMT_F32)
+      return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_F32, Geo<2, 2>>(mars, caution);
     // fp32 parameters and gradients over narrow moments (storage_dtype="bfloat16", ecc="bf16+8")
-    if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_BF16) return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_BF16>(mars, caution);
-    if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_ECC_BF16_8) return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_ECC_BF16_8>(mars, caution);
+    if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_BF16)
+      return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_BF16, Geo<2, 4>>(mars, caution);
+    if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_ECC_BF16_8)
+      return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_ECC_BF16_8, Geo<4, 1>>(mars, caution);
   }
   return pick_pass<ALGO, kDyn, kDyn, kDyn>(mars, caution);
 }
