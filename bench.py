@@ -147,8 +147,10 @@ def bench_first_order(cfg_name, steps, warmup, kernel_launches, rounding="philox
         params.append(p)
     opt = getattr(heavyball_amd, cls_name)(params, **kwargs)
     opt.rounding = rounding
-    # gradient sets resident in HBM before the timed region; cycled if memory is tight
-    n_sets = 4 if total < 1_000_000_000 else 1
+    # gradient sets resident in HBM before the timed region, cycled.  Two even for the 8B-shaped set (16 GB each): with one set
+    # every step would see the gradient of the step before, MARS' correction would vanish and caution's count pass would never
+    # meet an element that is too close to call
+    n_sets = 4 if total < 1_000_000_000 else 2
     grad_sets = [[(torch.randn(s, device=dev) * gstd).to(gdtype) for s in shapes] for _ in range(n_sets)]
 
     def one_step(k):

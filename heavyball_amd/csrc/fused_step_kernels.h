@@ -154,7 +154,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
       raw_decode<GF>(rg[k], gf, g);
     }
     if constexpr (kLazy) {
-      bool need = false;
+      uint32_t undecided = 0;  // bit j: element j is too close to call from the primaries
       uint32_t fast = 0;
       // Bounds, all on the safe side.  A bf16 + int8 pair lies within 2^(max(e, 1) - 135) of its primary x (e its exponent
       // field), which is at most max(|x| 2^-8, 2^-126) <= |x| 2^-8 + 2^-126: with x times a coefficient already at hand
@@ -183,15 +183,38 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
         const float em = __builtin_fabsf(s1) * k_ulp + k_a1 * dg + (__builtin_fabsf(s1) + __builtin_fabsf(s2)) * 0x1p-21f + c_m;
         sure = sure && __builtin_fabsf(mn) > em;  // NaN compares false: the exact route decides
         const bool inside = FULL || e + j < valid;
-        need = need || (inside && !sure);
-        fast += (inside && ((f2u(gs) ^ f2u(mn)) >> 31) != 0) ? 1u : 0u;
+        if (inside && !sure) undecided |= 1u << j;
+        else fast += (inside && ((f2u(gs) ^ f2u(mn)) >> 31) != 0) ? 1u : 0u;
       }
-      if (!need) {
-        masked += fast;
-        return;
+      masked += fast;
+      // The exact route, element by element: 0.2-0.3 % of the elements of a training-like state need it, which still is
+      // three quarters of the wavefronts (64 lanes of 8 elements), so it has to cost a wavefront little: one quartet's random
+      // numbers and the flagged elements alone, not the whole group with every lane but one idle.
+      if (undecided) {
+#pragma unroll
+        for (int q = 0; q < kE / 4; ++q) {
+          if (!(undecided & (0xFu << (4 * q)))) continue;
+          Rand8 r{{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u}};
+          if (MARS && a.rng.mode == HB_RNG_PHILOX) r = a.rng.call(idx + 4 * q, HB_STREAM_MARS_SR >> 1);
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            const int j = 4 * q + jj;
+            if (!((undecided >> j) & 1u)) continue;
+            const uint32_t hm = (rm[k].a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
+            const float mx = ecc_decode<true, true>(hm, (int)ld_as<int8_t>(a.m_corr + idx + j));
+            float gc = g[j];
+            if (MARS) {
+              const uint32_t ho = (ro[k].a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
+              const float ox = ecc_decode<true, true>(ho, (int)ld_as<int8_t>(a.og_corr + idx + j));
+              gc = g[j] * a.omamars + ox * a.amars;  // heavyball/utils.py:1048, then its rounding to the gradient's bf16
+              gc = bf16_to_f32(sr_bf16(gc, (r.w[jj >> 1] >> ((jj & 1) * 16)) & 0xFFFFu));  // word and half of HB_STREAM_MARS_SR
+            }
+            const float mn = mx * a.oma1 + gc * a.a1;  // heavyball/utils.py:1939; the sign of m / den is the sign of m
+            masked += ((f2u(gc) ^ f2u(mn)) >> 31) != 0 ? 1u : 0u;
+          }
+        }
       }
-      ld_slab<kE>(a.m_corr + idx, rm[k].c);
-      if (MARS) ld_slab<kE>(a.og_corr + idx, ro[k].c);
+      return;
     }
     raw_decode<SF>(rm[k], sf, m);
     if (kNeedV) raw_decode<SF>(rv[k], sf, v);
@@ -340,8 +363,14 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   }
 }
 
+#ifndef HB_COUNT_WAVES  // wavefronts per SIMD the compiler must leave room for (its register budget) in the count pass ...
+#define HB_COUNT_WAVES 1
+#endif
+#ifndef HB_STEP_WAVES  // ... and in the passes that write
+#define HB_STEP_WAVES 1
+#endif
 template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF, class GEO>
-__global__ __launch_bounds__(kThreads) void fused_step_kernel(const StepArgs a) {
+__global__ __launch_bounds__(kThreads, CAUTION == kCautionCount ? HB_COUNT_WAVES : HB_STEP_WAVES) void fused_step_kernel(const StepArgs a) {
   constexpr int kWork = GEO::kWork, kSub = GEO::kSub;
   const int pf = PF == kDyn ? a.pf : PF;
   const int gf = GF == kDyn ? a.gf : GF;
