@@ -204,3 +204,145 @@ def test_soap_products_and_orthonormalisation_at_full_size():
     assert torch.equal(GG, GG.T)  # both triangles accumulate the same products in the same order
     want = G.double().T[:4] @ G.double()
     assert torch.allclose(GG[:4].double(), want, rtol=1e-5, atol=1e-6 * want.abs().max().item())  # sums of 2048 cancelling products
+
+
+@pytest.mark.timeout(600)
+def test_muon_step_on_llama_sized_matrices_matches_oracle():
+    """``Muon.step()`` end to end (momentum, grouped Newton-Schulz on the 256-wide tile class, ``update_param_``) on a [1024, 4096]
+    and a [4096, 4096] matrix plus a vector, two steps against the oracle: the momentum bit for bit, the vector's parameter bit
+    for bit, each matrix' step to the Newton-Schulz tolerance (2e-2 relative Frobenius)."""
+    from oracle import muon as omuon
+    from oracle.rounding import HalfRounding
+
+    shapes = [(1024, 4096), (4096,), (4096, 4096)]
+    host, params = H.make_params(shapes, DEV)
+    kwargs = dict(betas=(0.95, 0.99), weight_decay=0.01, lr=0.02)
+    opt = heavyball_amd.Muon(params, **kwargs)
+    opt.rounding = "half"
+    orc = omuon.MuonOracle([h.clone() for h in host], rounding=HalfRounding(), **kwargs)
+    for k in (1, 2):
+        print("case step", k, flush=True)
+        grads = H.make_grads(shapes, k, torch.float32, 1e-2)
+        prev = [p.detach().cpu().clone() for p in params]
+        prev_o = [p.clone() for p in orc.params]
+        for p, g in zip(params, grads):
+            p.grad = g.to(DEV)
+        opt.step()
+        orc.step([g.clone() for g in grads])
+        torch.cuda.synchronize()
+        for i, p in enumerate(params):
+            H.assert_bit_equal(opt.state[p][0][opt.KEY], orc.state[i][orc.KEY], f"step {k} momentum {i}")
+            if p.dim() < 2:
+                H.assert_bit_equal(p.data, orc.params[i], f"step {k} vector {i}")
+                continue
+            got, want = (p.detach().cpu() - prev[i]).double(), (orc.params[i] - prev_o[i]).double()
+            err = ((got - want).norm() / want.norm()).item()
+            print(tuple(p.shape), "step vs oracle, rel fro", err, flush=True)
+            assert err < 2e-2, (k, i, err)
+
+
+@pytest.mark.timeout(900)
+def test_soap_with_both_factors_at_benchmark_shapes():
+    """The SOAP benchmark configuration as stated (max_precond_dim = 8192: every side of [2048, 2048], [2048, 8192] and
+    [8192, 2048] has a factor and a basis) through ``SOAP.step()``: initialisation, a step with a basis refresh and a plain step
+    in the refreshed basis (precondition_frequency = 2).  A float64 eigh of an 8192-wide factor on the CPU would take minutes,
+    so every step is checked through what it must satisfy, recomputed on the device in float64 from the optimizer's own state:
+
+      * the bases after initialisation are orthonormal and diagonalise their factors, eigenvalues in descending order;
+      * a step is Adam in the basis the step began with, rotated back: the parameters move by exactly that update, the second
+        moment is the one Adam leaves, the factors are the lerp of the old ones with G G^T and G^T G;
+      * a refreshed basis is orthonormal, it is the QR factor of (factor x old basis) with its columns sorted by the estimates
+        diag(Q^T GG Q) - checked as: new_basis^T (GG Q)[sorted] is upper triangular, up to exchanges of neighbouring columns
+        whose sort keys fp32 cannot tell apart - it diagonalises the factor no worse than the old one, and exp_avg is the
+        momentum of the step rotated from the old basis into the new one."""
+    from heavyball_amd.optim import beta_debias, f32
+
+    shapes = [(2048, 2048), (2048, 8192), (8192, 2048)]
+    free, _ = torch.cuda.mem_get_info(DEV)
+    if free < 40 * 2**30:
+        pytest.skip("needs 40 GiB of device memory")
+    host, params = H.make_params(shapes, DEV)
+    lr, wd, b1, b2, sb, eps = 3e-3, 0.01, 0.9, 0.95, 0.95, 1e-8
+    opt = heavyball_amd.SOAP(params, lr=lr, betas=(b1, b2), shampoo_beta=sb, eps=eps, weight_decay=wd, precondition_frequency=2,
+                             max_precond_dim=8192)  # fmt: skip
+    KM, KV, KQ, KGG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
+
+    def rel(a, b):
+        return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-300)).item()
+
+    def orthonormal(q):
+        qd = q.double()
+        return (qd.T @ qd - torch.eye(qd.shape[0], dtype=torch.float64, device=DEV)).abs().max().item()
+
+    fired = []
+    for k in (1, 2, 3):
+        print("case step", k, flush=True)
+        grads = [g.to(DEV) for g in H.make_grads(shapes, k, torch.float32, 1e-2)]
+        before = []
+        for p in params:
+            st = opt.state[p][0] if p in opt.state and KM in opt.state[p].get(0, {}) else None
+            before.append(None if st is None else dict(p=p.detach().clone(), m=st[KM][0].clone(), v=st[KV][0].clone(),
+                                                       Q=[q[0].clone() for q in st[KQ]], GG=[m[0].clone() for m in st[KGG]]))  # fmt: skip
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.step()
+        torch.cuda.synchronize()
+        fired.append(bool(opt.param_groups[0]["is_preconditioning"]))
+        for i, (p, g) in enumerate(zip(params, grads)):
+            st = opt.state[p][0]
+            G = g.double()
+            if k == 1:
+                assert torch.equal(p.detach().cpu(), host[i])  # the first step only initialises
+                for li, (q, gg) in enumerate(zip(st[KQ], st[KGG])):
+                    want = G @ G.T if li == 0 else G.T @ G  # beta = 0 at initialisation: the factor is the product itself
+                    assert rel(gg[0], want) < 1e-5, (i, li)
+                    assert orthonormal(q[0]) < 1e-4
+                    lam = q[0].double().T @ gg[0].double() @ q[0].double()
+                    top = lam.diagonal().max().item()
+                    assert (lam - torch.diag(lam.diagonal())).abs().max().item() < 1e-4 * top, (i, li)
+                    assert (lam.diagonal()[1:] - lam.diagonal()[:-1]).max().item() < 1e-4 * top, (i, li)
+                continue
+            b = before[i]
+            Ql, Qr = b["Q"][0].double(), b["Q"][1].double()
+            step = torch.tensor(k, dtype=torch.int64)
+            d1, d2 = float(beta_debias(f32(b1), step - 1)), float(beta_debias(f32(b2), step - 1))  # heavyball/chainable.py:1270
+            gp = Ql.T @ G @ Qr
+            m_new = b["m"].double() * d1 + gp * (1 - d1)
+            v_new = b["v"].double() * d2 + gp * gp * (1 - d2)
+            precond = m_new / v_new.sqrt().clamp(min=eps)
+            update = Ql @ precond @ Qr.T
+            want_p = b["p"].double() * (1 - wd * lr) - lr * update
+            moved, want_moved = p.detach().double() - b["p"].double(), want_p - b["p"].double()
+            assert rel(moved, want_moved) < 2e-3, (k, i, rel(moved, want_moved))
+            assert rel(st[KV][0], v_new) < 1e-4, (k, i)
+            a = 1 - float(beta_debias(sb, step))  # heavyball/chainable.py:1244
+            for li, gg in enumerate(st[KGG]):
+                outer = G @ G.T if li == 0 else G.T @ G
+                assert rel(gg[0], b["GG"][li].double() * (1 - a) + outer * a) < 1e-5, (k, i, li)
+            if not fired[-1]:
+                assert rel(st[KM][0], m_new) < 1e-4, (k, i)
+                for li, q in enumerate(st[KQ]):
+                    assert torch.equal(q[0], b["Q"][li])
+                continue
+            new_q = [q[0].double() for q in st[KQ]]
+            for li, qn in enumerate(new_q):
+                assert orthonormal(st[KQ][li][0]) < 1e-4, (k, i, li)
+                old = b["Q"][li].double()
+                tmp = st[KGG][li][0].double() @ old
+                order = torch.argsort((old * tmp).sum(0), descending=True)
+                # upper triangular if qn[:, order] is the QR factor of tmp[:, order].  Thousands of sort keys lie closer together
+                # than fp32 products resolve, so the optimizer's order is this float64 order up to exchanges among neighbours:
+                # the triangle is asked for outside a band of 64 columns, and inside the band only to the size of the
+                # neighbouring diagonal entries
+                r = qn[:, order].T @ tmp[:, order]
+                scale = r.diagonal().abs().max().item()
+                assert r.tril(-64).abs().max().item() < 1e-4 * scale, (k, i, li, r.tril(-64).abs().max().item() / scale)
+                assert r.tril(-1).abs().max().item() < 2e-2 * scale, (k, i, li, r.tril(-1).abs().max().item() / scale)
+                # and one step of power iteration cannot make the basis diagonalise its factor worse
+                def off_mass(q):
+                    lam = q.T @ st[KGG][li][0].double() @ q
+                    return (lam - torch.diag(lam.diagonal())).norm().item()
+                assert off_mass(qn) <= off_mass(old) * 1.001, (k, i, li)
+            want_m = new_q[0].T @ (Ql @ m_new @ Qr.T) @ new_q[1]  # heavyball/utils.py:877-884
+            assert rel(st[KM][0], want_m) < 2e-3, (k, i, rel(st[KM][0], want_m))
+    assert fired == [False, True, False]
