@@ -440,14 +440,19 @@ StepKernel pick_algo(bool mars, int caution, int pf, int gf, int sf) {
     return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_ECC_BF16_8>(mars, caution);
   if (pf == HB_FMT_ECC_BF16_8 && gf == HB_FMT_BF16 && sf == HB_FMT_ECC_BF16_8)
     return pick_pass<ALGO, HB_FMT_ECC_BF16_8, HB_FMT_BF16, HB_FMT_ECC_BF16_8>(mars, caution);
-  // mixed-precision set-ups without ECC, for the two optimizers they are mostly run with: bf16 parameters and gradients over
-  // fp32 or bf16 moments, fp32 parameters with bf16 gradients (measured 4.6 / 3.3 / 5.2 TB/s on the run-time-format kernel)
+  // mixed-precision set-ups without ECC: bf16 parameters and gradients over fp32 moments, fp32 parameters with bf16 gradients
+  // (measured 4.6 / 5.2 TB/s on the run-time-format kernel), for every algorithm
+  if (pf == HB_FMT_BF16 && gf == HB_FMT_BF16 && sf == HB_FMT_F32)
+    return pick_pass<ALGO, HB_FMT_BF16, HB_FMT_BF16, HB_FMT_F32, Geo<4, 1>>(mars, caution);
+  if (pf == HB_FMT_F32 && gf == HB_FMT_BF16 && sf == HB_FMT_F32)
+    return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_F32, Geo<2, 2>>(mars, caution);
+  // for the two optimizers that are mostly run: bf16 moments, and the wide correction of the bf16 ECC pair
   if constexpr (ALGO == HB_ALGO_ADAM || ALGO == HB_ALGO_LAPROP) {
-    if (pf == HB_FMT_BF16 && gf == HB_FMT_BF16 && sf == HB_FMT_F32)
-      return pick_pass<ALGO, HB_FMT_BF16, HB_FMT_BF16, HB_FMT_F32, Geo<4, 1>>(mars, caution);
     if (pf == HB_FMT_BF16 && gf == HB_FMT_BF16 && sf == HB_FMT_BF16) return pick_pass<ALGO, HB_FMT_BF16, HB_FMT_BF16, HB_FMT_BF16>(mars, caution);
-    if (pf == HB_FMT_F32 && gf == HB_FMT_BF16 && sf == HB_FMT_F32)
-      return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_F32, Geo<2, 2>>(mars, caution);
+    if (pf == HB_FMT_F32 && gf == HB_FMT_BF16 && sf == HB_FMT_ECC_BF16_16)
+      return pick_pass<ALGO, HB_FMT_F32, HB_FMT_BF16, HB_FMT_ECC_BF16_16>(mars, caution);
+    if (pf == HB_FMT_ECC_BF16_16 && gf == HB_FMT_BF16 && sf == HB_FMT_ECC_BF16_16)
+      return pick_pass<ALGO, HB_FMT_ECC_BF16_16, HB_FMT_BF16, HB_FMT_ECC_BF16_16>(mars, caution);
     // fp32 parameters and gradients over narrow moments (storage_dtype="bfloat16", ecc="bf16+8")
     if (pf == HB_FMT_F32 && gf == HB_FMT_F32 && sf == HB_FMT_BF16)
       return pick_pass<ALGO, HB_FMT_F32, HB_FMT_F32, HB_FMT_BF16, Geo<2, 4>>(mars, caution);
