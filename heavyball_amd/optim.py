@@ -849,8 +849,6 @@ class FirstOrder(HBOptimizer):
     def _run_group(self, gi, group, active):
         narrow = not self.promote and any(g.dtype != torch.float32 for _, g in active)
         unfused = self.update_clipping is not None or (self._unfused_for_narrow_grads and narrow)
-        if unfused and any(g.dtype == torch.float16 for _, g in active) and not self.promote:
-            raise NotImplementedError("the un-fused chain (update_clipping, MuonAdamW's vector route) with float16 gradients")
         L = _lib.lib()
         step = group["step"]
         lr = f32(group["lr"])
@@ -1008,6 +1006,11 @@ class FirstOrder(HBOptimizer):
                     _lib.check(L.hb_sr_bf16(wide.data_ptr(), narrow.data_ptr(), wide.numel(), self._rng_mode(), self.rng_seed,
                                             int(step) & 0xFFFFFFFF, _lib.STREAM_UPDATE_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
                 upd_role, upd_fmt = "_update16", _lib.FMT_BF16
+            elif gdt == torch.float16 and self.update_clipping is not None:
+                # a float16 update buffer takes the clipped values through a plain cast (heavyball/utils.py:2363-2370 rounds
+                # stochastically into bfloat16 only); the values stay in the fp32 role, every one of them a float16 number
+                wide = b.slab.role("_update", torch.float32)
+                wide.copy_(wide.to(torch.float16))
             offsets, numel = b.slab.meta()
             chunks, n_chunks = b.slab.chunks(tuple(i for i, _ in lst))
             ptrs = [0] * len(b.params)

@@ -331,6 +331,16 @@ def make_both_clips():
              grad_scale=1.0)  # fmt: skip
 
 
+def make_fp16_unfused():
+    """float16 gradients on the un-fused chain (heavyball/chainable.py:2676-2701): the update buffer is float16, every write into
+    it (the transform's result, the clip's) is a plain cast, and the tail compares it with the float16 gradient."""
+    shapes = [(4, 8), (16,), (3, 5)]
+    run_traj("adamw_updclip_l2_fp16grad", heavyball.AdamW, dict(update_clipping="l2_clip_", weight_decay=0.01), shapes, torch.float16, 4)
+    run_traj("laprop_updclip_rms_mars_fp16grad_ecc_caution", heavyball.LaProp, dict(update_clipping="rmsnorm_clip_", mars=True, ecc="bf16+8",
+                                                                                   caution=True, lr=0.01), shapes, torch.float16, 4)  # fmt: skip
+    run_traj("adopt_updclip_global_l2_fp16grad", heavyball.ADOPT, dict(update_clipping="global_l2norm_clip"), shapes, torch.float16, 5)
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -488,7 +498,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -505,6 +515,8 @@ if __name__ == "__main__":
         make_clip_combinations()
     if "bothclips" in which:
         make_both_clips()
+    if "fp16unfused" in which:
+        make_fp16_unfused()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:

@@ -433,6 +433,16 @@ CLIP_COMBOS = [
     ("nadam_updclip_rms_coupled_wd", "NAdam", dict(update_clipping="rmsnorm_clip_", weight_decay=0.01), torch.float32, 1e-2),
     ("nadam_updclip_l2_decoupled_caution_bf16grad", "NAdam", dict(update_clipping="l2_clip_", weight_decay=0.01, decoupled_weight_decay=True,
                                                                   caution=True), torch.bfloat16, 1e-2),
+    # float16 gradients: the update buffer is float16, written by plain casts
+    ("adamw_updclip_l2_fp16grad", "AdamW", dict(update_clipping="l2_clip_", weight_decay=0.01), torch.float16, 1e-2),
+    ("laprop_updclip_rms_mars_ecc_caution_fp16grad", "LaProp", dict(update_clipping="rmsnorm_clip_", mars=True, ecc="bf16+8", caution=True, lr=0.01),
+     torch.float16, 1e-2),
+    ("adopt_updclip_global_l2_fp16grad", "ADOPT", dict(update_clipping="global_l2norm_clip"), torch.float16, 1e-2),
+    # MARS, both clips and caution in one chain: the tail's sign test reads the MARS-corrected gradient
+    ("adamw_mars_both_clips_caution", "AdamW", dict(mars=True, gradient_clipping="l2_clip_", update_clipping="rmsnorm_clip_", caution=True,
+                                                    weight_decay=0.01, mars_gamma=0.5), torch.float32, 1.0),
+    ("laprop_mars_both_clips_caution_bf16grad_ecc", "LaProp", dict(mars=True, gradient_clipping="global_l2norm_clip", update_clipping="l2_clip_",
+                                                                   caution=True, ecc="bf16+8", mars_gamma=0.5, lr=0.01), torch.bfloat16, 1.0),
 ]
 
 
@@ -448,7 +458,7 @@ def test_clipping_combinations_match_oracle(case):
     print("case", name, flush=True)
     cls, kind = CLS[cls_name]
     host, params, opt, orc = H.build_pair(cls, kind, RAGGED, kwargs, DEV, rounding="philox")
-    bf16_update = gdt == torch.bfloat16 and "update_clipping" in kwargs
+    bf16_update = gdt in (torch.bfloat16, torch.float16) and "update_clipping" in kwargs  # a 16-bit update buffer
     for k in range(1, 5):
         grads = H.make_grads(RAGGED, k, gdt, gscale)
         for p, g in zip(params, grads):
@@ -462,7 +472,7 @@ def test_clipping_combinations_match_oracle(case):
             want = {"param": pw.primary if hasattr(pw, "primary") else pw,
                     **{kk: v for kk, v in orc.state[i].items() if kk != "step" and isinstance(v, torch.Tensor)}}
             got = {"param": p.data, **st}
-            if not (bf16_update or gdt == torch.bfloat16):
+            if not (bf16_update or gdt in (torch.bfloat16, torch.float16)):
                 H.assert_close_in_scale(got, want, f"{name} step {k} tensor {i}")
                 continue
             for key, w in want.items():
@@ -482,9 +492,11 @@ def test_clipping_combinations_match_oracle(case):
 
 def test_clipping_combinations_that_are_not_built_raise():
     p = [torch.nn.Parameter(torch.zeros(8, device=DEV))]
+    p.append(torch.nn.Parameter(torch.zeros(8, device=DEV)))
     opt = heavyball_amd.AdamW(p, update_clipping="l2_clip_")
-    p[0].grad_dtype = None
-    p[0].grad = torch.ones(8, device=DEV, dtype=torch.float16)  # float16 gradients with update_clipping are not built
+    p[0].grad_dtype = p[1].grad_dtype = None
+    p[0].grad = torch.ones(8, device=DEV, dtype=torch.bfloat16)  # gradients of two dtypes in one bucket under a clip are not built
+    p[1].grad = torch.ones(8, device=DEV)
     with pytest.raises(NotImplementedError):
         opt.step()
     with pytest.raises(ValueError):
