@@ -101,6 +101,9 @@ class Muon(HBOptimizer):
         return parts
 
     def _run_group(self, gi, group, active):
+        self._run_gen(self._run_group_gen(gi, group, active))
+
+    def _run_group_gen(self, gi, group, active):
         active = [(p, g) for p, g in active if p.numel() > 0]  # an empty tensor has nothing to orthogonalise or update
         if not active:
             return
@@ -187,7 +190,7 @@ class Muon(HBOptimizer):
                 if gdt not in (torch.float32, torch.bfloat16):
                     raise NotImplementedError(f"mars with {gdt} gradients on the Muon path")
                 self._mars_prologue(L, group, b, lst, gdt, step, mars_a, mars_oma, mom_fmt, k_o)
-            for (b, _, gdt), res in zip(work, self._clip_gradients(L, group, work, step, gathered=mars)):
+            for (b, _, gdt), res in zip(work, (yield from self._clip_gradients_gen(L, group, work, step, gathered=mars))):
                 clipped[(id(b), gdt)] = res
         if self.update_clipping is not None and any(g.dtype != torch.float32 for _, g in active) and not self.promote:
             raise NotImplementedError("update_clipping with 16-bit gradients (the reference rounds the clipped update to their dtype)")
@@ -247,7 +250,7 @@ class Muon(HBOptimizer):
                     _lib.check(L.hb_ns5_batched_mixed(n, ptrs, ptrs, rows_a, cols_a, arr, flag_a, 1e-7, scale, self._rng_mode(), self.rng_seed,
                                                       int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream), "hb_ns5_batched_mixed")  # fmt: skip
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group
-            keep.append(self._clip_updates(L, [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared]))
+            keep.append((yield (self.update_clipping, "_update", [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared])))
         for b, items, by_dtype in prepared:
             offsets, numel = b.slab.meta()
             stream = current_stream_ptr(b.device)
@@ -288,8 +291,8 @@ class MuonAdamW(Muon, FirstOrder):
     State names and initialisation sets follow the reference's index walk with the route in place
     (``nesterov_ema_momentum_4`` with {2, 3, 4}, ``exp_avg_exp_avg_4`` under ``nesterov=False``; ``scale_by_adam_exp_avg_0`` /
     ``_exp_avg_sq_0`` with {0}; ``mars_mars_old_grad_6`` and a 6 in both sets under ``mars``).  ``ecc`` / ``storage_dtype`` apply
-    to the state of both routes.  ``gradient_clipping`` / ``update_clipping`` take the per-tensor kinds (``l2_clip_``,
-    ``rmsnorm_clip_``); a norm over the whole group would span the two routes and raises NotImplementedError.
+    to the state of both routes.  ``gradient_clipping`` / ``update_clipping`` act on the tensors of both routes at once, as the
+    reference's chain places them around the route: a norm over the whole group is one norm over matrices and vectors.
     """
 
     KEY = "nesterov_ema_momentum_4"
@@ -311,9 +314,6 @@ class MuonAdamW(Muon, FirstOrder):
                          param_ecc=param_ecc, orig_shapes=orig_shapes, **kwargs)  # fmt: skip
         if not nesterov:  # heavyball/__init__.py:527-529: exp_avg heads the matrix route instead
             self.KEY = "exp_avg_exp_avg_4"
-        for kind in (self.gradient_clipping, self.update_clipping):
-            if kind is not None and kind.startswith("global_"):
-                raise NotImplementedError("MuonAdamW: clipping by a norm over the whole group (it would span both routes)")
         for group in self.param_groups:  # the reference's MuonAdamW has no such argument (heavyball/__init__.py:499-523)
             group.pop("heavyball_momentum", None)
         self.defaults.pop("heavyball_momentum", None)
@@ -322,12 +322,16 @@ class MuonAdamW(Muon, FirstOrder):
         return 1 if p.ndim >= 2 else 0
 
     def _run_group(self, gi, group, active):
+        # the two routes side by side: a clip (heavyball/chainable.py:2696-2701 puts both clips around the route) acts on the
+        # tensors of both at once, so a norm over the whole group spans matrices and vectors
         matrices = [(p, g) for p, g in active if p.ndim >= 2]
         vectors = [(p, g) for p, g in active if p.ndim < 2]
+        gens = []
         if matrices:
-            Muon._run_group(self, gi, group, matrices)
+            gens.append(Muon._run_group_gen(self, gi, group, matrices))
         if vectors:
-            FirstOrder._run_group(self, gi, group, vectors)
+            gens.append(FirstOrder._run_group_gen(self, gi, group, vectors))
+        self._run_gens(gens)
 
 
 class SplitOpt:

@@ -538,9 +538,46 @@ class HBOptimizer(torch.optim.Optimizer):
             _lib.check(L.hb_fused_step(d, current_stream_ptr(b.device)), "hb_fused_step (MARS prologue)")
         self._last_launch = (d, (table, chunks, offsets, numel))
 
+    def _run_gen(self, gen):
+        """Runs a step generator to its end.  Such a generator yields ``(clip kind, slab role, [(bucket, tensor indices)])`` wherever
+        the chain clips by a norm, and is sent back what ``_clip_role`` returns; its own return value is handed on."""
+        L = _lib.lib()
+        try:
+            req = next(gen)
+            while True:
+                req = gen.send(self._clip_role(L, req[0], req[1], req[2]))
+        except StopIteration as done:
+            return done.value
+
+    def _run_gens(self, gens):
+        """Several step generators side by side (the routes of one parameter group): they reach their clip points in the same
+        order, and each point is clipped once over the tensors of all of them, so that a norm over the whole group is one norm."""
+        L = _lib.lib()
+        waiting = []
+        for g in gens:
+            try:
+                waiting.append((g, next(g)))
+            except StopIteration:
+                pass
+        while waiting:
+            kind, role = waiting[0][1][0], waiting[0][1][1]
+            if any(r[0] != kind or r[1] != role for _, r in waiting):
+                raise _lib.HbError("the routes of a parameter group reached different clip points")
+            keep = self._clip_role(L, kind, role, [bk for _, r in waiting for bk in r[2]])
+            nxt = []
+            for g, _ in waiting:
+                try:
+                    nxt.append((g, g.send(keep)))
+                except StopIteration:
+                    pass
+            waiting = nxt
+
     def _clip_gradients(self, L, group, buckets, step, gathered=False):
+        return self._run_gen(self._clip_gradients_gen(L, group, buckets, step, gathered))
+
+    def _clip_gradients_gen(self, L, group, buckets, step, gathered=False):
         """``gradient_clipping`` (heavyball/chainable.py:2696-2699): the gradients of the group are gathered into the fp32
-        slab role ``_clip``, clipped there (``_clip_role``) and, for bf16 gradients, rounded back to bf16 the way
+        slab role ``_clip``, clipped there (a clip point, see ``_run_gen``) and, for bf16 gradients, rounded back to bf16 the way
         ``copy_stochastic_`` does (``hb_sr_bf16``).  ``buckets``: [(bucket, [(index, gradient)], gradient dtype)].  Returns,
         per bucket, the slab role and format the step then reads its gradients from.  Three extra passes over the
         gradients: a capability, not a tuned path."""
@@ -553,7 +590,7 @@ class HBOptimizer(torch.optim.Optimizer):
                     b.slab.view("_clip", i).copy_(g)
         keep = None
         if self.gradient_clipping is not None:  # None: the caller only wants the gathered role in the gradients' dtype
-            keep = self._clip_role(L, self.gradient_clipping, "_clip", [(b, [i for i, _ in lst]) for b, lst, _ in buckets])
+            keep = yield (self.gradient_clipping, "_clip", [(b, [i for i, _ in lst]) for b, lst, _ in buckets])
         result = []
         for b, lst, gdt in buckets:
             role = b.slab.role("_clip", torch.float32)
@@ -847,6 +884,9 @@ class FirstOrder(HBOptimizer):
     _unfused_for_narrow_grads = False
 
     def _run_group(self, gi, group, active):
+        self._run_gen(self._run_group_gen(gi, group, active))
+
+    def _run_group_gen(self, gi, group, active):
         narrow = not self.promote and any(g.dtype != torch.float32 for _, g in active)
         unfused = self.update_clipping is not None or (self._unfused_for_narrow_grads and narrow)
         L = _lib.lib()
@@ -921,9 +961,9 @@ class FirstOrder(HBOptimizer):
             flags &= ~(_lib.FLAG_MARS | _lib.FLAG_WRITE_GRAD)
             mars = False
             prologue = True
-            clipped = self._clip_gradients(L, group, work, step, gathered=True)
+            clipped = yield from self._clip_gradients_gen(L, group, work, step, gathered=True)
         elif self.gradient_clipping is not None:
-            clipped = self._clip_gradients(L, group, work, step)
+            clipped = yield from self._clip_gradients_gen(L, group, work, step)
         else:
             clipped = [None] * len(work)
         plannable = (as_given and not unfused and self.gradient_clipping is None and not self._use_palm and self._plannable
@@ -995,7 +1035,9 @@ class FirstOrder(HBOptimizer):
             self._plans[gi] = plan
         if not unfused:
             return
-        keep = self._clip_updates(L, [(b, [i for i, _ in lst]) for b, lst, _ in work]) if self.update_clipping is not None else None
+        keep = None
+        if self.update_clipping is not None:
+            keep = yield (self.update_clipping, "_update", [(b, [i for i, _ in lst]) for b, lst, _ in work])
         decay_py = group["weight_decay"]  # update_param_ keeps decay a python float (heavyball/utils.py:2393-2406)
         for (b, lst, gdt), clip in zip(work, clipped):
             upd_role, upd_fmt = "_update", _lib.FMT_F32

@@ -325,6 +325,35 @@ def global_rmsnorm_clip(xs: List[Tensor], clip_at=1.0, eps=1e-8) -> List[Tensor]
     return [promote(x) * scalar for x in xs]
 
 
+def run_clip_points(gens):
+    """Runs step generators side by side.  Each yields ``(clip kind, tensors, tensor indices)`` where the reference's chain clips
+    (heavyball/chainable.py:2696-2701) and is sent its tensors back clipped.  The generators of one parameter group (the two routes
+    of MuonAdamW) reach their clip points in the same order, and each point is clipped once over the tensors of all of them, in the
+    order of the group's parameters: the reference's chain places the clips around the route."""
+    fns = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip, "global_rmsnorm_clip": global_rmsnorm_clip}
+    waiting = []
+    for g in gens:
+        try:
+            waiting.append((g, next(g)))
+        except StopIteration:
+            pass
+    while waiting:
+        kind = waiting[0][1][0]
+        assert all(r[0] == kind for _, r in waiting)
+        merged = sorted(((t, k, j) for k, (_, r) in enumerate(waiting) for j, t in enumerate(r[2])))
+        out = fns[kind]([waiting[k][1][1][j] for _, k, j in merged])
+        back = [[None] * len(r[1]) for _, r in waiting]
+        for (_, k, j), c in zip(merged, out):
+            back[k][j] = c
+        nxt = []
+        for (g, _), b in zip(waiting, back):
+            try:
+                nxt.append((g, g.send(b)))
+            except StopIteration:
+                pass
+        waiting = nxt
+
+
 # ---------------------------------------------------------------------------------------------------------
 # The step loop of one param group
 # ---------------------------------------------------------------------------------------------------------
@@ -439,6 +468,10 @@ class FirstOrderOracle:
         return EccTensor(st[k], st[k + "::ecc"])
 
     def step(self, grads: List[Optional[Tensor]]):
+        run_clip_points([self.step_gen(grads)])
+
+    def step_gen(self, grads: List[Optional[Tensor]]):
+        """The step as a generator: it yields ``(clip kind, tensors)`` at the chain's clip points and is sent the clipped tensors."""
         idx = [i for i, g in enumerate(grads) if g is not None]
         if not idx:
             return
@@ -460,9 +493,8 @@ class FirstOrderOracle:
         if self.gradient_clipping is not None:
             # heavyball/chainable.py:2696-2699: the clip acts on the update after MARS and before the Adam/LaProp transform;
             # heavyball/utils.py:3226-3232 writes x32 * scale back with copy_stochastic_ (a stochastic round for bf16)
-            fn = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip,
-                  "global_rmsnorm_clip": global_rmsnorm_clip}[self.gradient_clipping]  # fmt: skip
-            for j, (u, c) in enumerate(zip(update, fn(update))):
+            clipped = yield (self.gradient_clipping, update, idx)
+            for j, (u, c) in enumerate(zip(update, clipped)):
                 if u.dtype == torch.bfloat16:
                     u.copy_(stochastic_round(c, rounding.noise16(philox.STREAM_CLIP, idx[j], u.shape)))
                 else:
@@ -510,9 +542,8 @@ class FirstOrderOracle:
             for u, n, t in zip(update, new, idx):
                 copy_stochastic(u, n, rounding, philox.STREAM_UPDATE, t)
             if self.update_clipping is not None:
-                fn = {"l2_clip_": l2_clip, "rmsnorm_clip_": rmsnorm_clip, "global_l2norm_clip": global_l2norm_clip,
-                      "global_rmsnorm_clip": global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
-                for u, c, t in zip(update, fn(update), idx):
+                clipped = yield (self.update_clipping, update, idx)
+                for u, c, t in zip(update, clipped, idx):
                     copy_stochastic(u, c, rounding, philox.STREAM_UPDATE_CLIP, t)
             # the tail of the chain decays with the group's weight_decay whatever the transform did with it (NAdam: on top of its own)
             update_param_(p, update, lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)

@@ -161,6 +161,13 @@ class MuonOracle:
         return st[key] if self.ecc is None else EccTensor(st[key], st[key + "::ecc"])
 
     def step(self, grads):
+        from . import first_order as fo
+
+        fo.run_clip_points([self.step_gen(grads)])
+
+    def step_gen(self, grads):
+        """The step as a generator that yields ``(clip kind, tensors)`` where the chain clips (heavyball/chainable.py:2696-2701) and is
+        sent the clipped tensors back: a group with two routes (MuonAdamW) clips the tensors of both at once."""
         idx = [i for i, g in enumerate(grads) if g is not None]
         if not idx:
             return
@@ -179,11 +186,8 @@ class MuonOracle:
             for g_, u_ in zip(grad, update):
                 g_.copy_(u_)
         if self.gradient_clipping is not None:  # heavyball/chainable.py:2696-2699: on the update, ahead of the momentum
-            from . import first_order as fo
-
-            fn = {"l2_clip_": fo.l2_clip, "rmsnorm_clip_": fo.rmsnorm_clip, "global_l2norm_clip": fo.global_l2norm_clip,
-                  "global_rmsnorm_clip": fo.global_rmsnorm_clip}[self.gradient_clipping]  # fmt: skip
-            for j, (u, c) in enumerate(zip(update, fn(update))):
+            clipped = yield (self.gradient_clipping, update, idx)
+            for j, (u, c) in enumerate(zip(update, clipped)):
                 if u.dtype == torch.bfloat16:
                     u.copy_(stochastic_round(c, rounding.noise16(philox.STREAM_CLIP, idx[j], u.shape)))
                 else:
@@ -203,11 +207,7 @@ class MuonOracle:
             shape = u.shape
             out.append(orthogonal(u.flatten(1, -1), rounding, i, self.mode).reshape(shape))
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701 (fp32 updates: a plain copy back)
-            from . import first_order as fo
-
-            fn = {"l2_clip_": fo.l2_clip, "rmsnorm_clip_": fo.rmsnorm_clip, "global_l2norm_clip": fo.global_l2norm_clip,
-                  "global_rmsnorm_clip": fo.global_rmsnorm_clip}[self.update_clipping]  # fmt: skip
-            out = fn(out)
+            out = yield (self.update_clipping, out, idx)
         update_param_(p, out, lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)
 
 
@@ -222,8 +222,6 @@ class MuonAdamWOracle:
                  nesterov=True, gradient_clipping=None, update_clipping=None, param_ecc=None):  # fmt: skip
         from .first_order import FirstOrderOracle, narrow_params
 
-        for kind in (gradient_clipping, update_clipping):
-            assert kind in (None, "l2_clip_", "rmsnorm_clip_"), "a norm over the whole group would span both routes"
         self.params = params
         self.mat_idx = [i for i, p in enumerate(params) if p.dim() >= 2]
         self.vec_idx = [i for i, p in enumerate(params) if p.dim() < 2]
@@ -246,8 +244,12 @@ class MuonAdamWOracle:
     def step(self, grads):
         if all(g is None for g in grads):
             return
-        self.muon.step([g if i in self.mat_idx else None for i, g in enumerate(grads)])
-        self.adam.step([g if i in self.vec_idx else None for i, g in enumerate(grads)])
+        from . import first_order as fo
+
+        # both routes side by side: the clips sit around the route (heavyball/chainable.py:2696-2701), so each acts on the
+        # tensors of the whole group at once
+        fo.run_clip_points([self.muon.step_gen([g if i in self.mat_idx else None for i, g in enumerate(grads)]),
+                            self.adam.step_gen([g if i in self.vec_idx else None for i, g in enumerate(grads)])])  # fmt: skip
         # one step counter for the group (heavyball/chainable.py:2531-2570): keep the two halves aligned when one had no gradient
         top = max(int(self.muon.step_count), int(self.adam.step_count))
         self.muon.step_count = torch.tensor(top, dtype=torch.int64)

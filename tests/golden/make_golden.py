@@ -341,6 +341,17 @@ def make_fp16_unfused():
     run_traj("adopt_updclip_global_l2_fp16grad", heavyball.ADOPT, dict(update_clipping="global_l2norm_clip"), shapes, torch.float16, 5)
 
 
+def make_group_norms():
+    """MuonAdamW with clips by a norm over the whole group (heavyball/__init__.py:475-540, heavyball/chainable.py:2696-2701): the clips
+    sit around the route, so one norm spans the matrices of the Muon route and the vectors of the Adam route."""
+    shapes = [(8, 16), (16,), (24, 8), (4, 3, 6), (5,)]
+    run_traj("muonadamw_global_clips_caution", heavyball.MuonAdamW, dict(gradient_clipping="global_l2norm_clip", update_clipping="global_rmsnorm_clip",
+                                                                         caution=True, weight_decay=0.01, lr=0.02), shapes, torch.float32, 4,
+             grad_scale=1.0)  # fmt: skip
+    run_traj("muonadamw_mars_global_rms_gradclip", heavyball.MuonAdamW, dict(mars=True, gradient_clipping="global_rmsnorm_clip", weight_decay=0.01),
+             shapes, torch.float32, 4, grad_scale=3.0)  # fmt: skip
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -498,7 +509,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -517,6 +528,8 @@ if __name__ == "__main__":
         make_both_clips()
     if "fp16unfused" in which:
         make_fp16_unfused()
+    if "groupnorms" in which:
+        make_group_norms()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:
