@@ -192,8 +192,6 @@ class Muon(HBOptimizer):
                 self._mars_prologue(L, group, b, lst, gdt, step, mars_a, mars_oma, mom_fmt, k_o)
             for (b, _, gdt), res in zip(work, (yield from self._clip_gradients_gen(L, group, work, step, gathered=mars))):
                 clipped[(id(b), gdt)] = res
-        if self.update_clipping is not None and any(g.dtype != torch.float32 for _, g in active) and not self.promote:
-            raise NotImplementedError("update_clipping with 16-bit gradients (the reference rounds the clipped update to their dtype)")
         keep = []
         tables = {}  # (bucket, gradient dtype) -> device table of gradient pointers
         for b, items, by_dtype in prepared:
@@ -251,6 +249,13 @@ class Muon(HBOptimizer):
                                                       int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream), "hb_ns5_batched_mixed")  # fmt: skip
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group
             keep.append((yield (self.update_clipping, "_update", [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared])))
+            for b, items, by_dtype in prepared:
+                if torch.bfloat16 in by_dtype:
+                    # the clip writes its result back into the bf16 update buffer through copy_stochastic_ (heavyball/utils.py:3231)
+                    wide, narrow = b.slab.role("_update", torch.float32), b.slab.role("_update16", torch.bfloat16)
+                    with torch.cuda.device(b.device):
+                        _lib.check(L.hb_sr_bf16(wide.data_ptr(), narrow.data_ptr(), wide.numel(), self._rng_mode(), self.rng_seed,
+                                                int(step) & 0xFFFFFFFF, _lib.STREAM_UPDATE_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
         for b, items, by_dtype in prepared:
             offsets, numel = b.slab.meta()
             stream = current_stream_ptr(b.device)
@@ -268,6 +273,8 @@ class Muon(HBOptimizer):
                         # positive factor, which keeps every sign
                         d.grad, d.grad_ptrs, d.grad_fmt = b.slab.ptr("_clip"), None, _lib.FMT_F32
                     d.exp_avg = b.slab.ptr("_update")
+                    if self.update_clipping is not None and gdt == torch.bfloat16:
+                        d.exp_avg, d.state_fmt = b.slab.ptr("_update16"), _lib.FMT_BF16
                     d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
                     d.caution_count = b.caution_scratch().data_ptr() if group["caution"] else None
                     d.n_chunks, d.n_tensors = n_chunks, len(b.params)

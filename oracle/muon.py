@@ -206,8 +206,12 @@ class MuonOracle:
                 continue
             shape = u.shape
             out.append(orthogonal(u.flatten(1, -1), rounding, i, self.mode).reshape(shape))
-        if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701 (fp32 updates: a plain copy back)
-            out = yield (self.update_clipping, out, idx)
+        if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701
+            clipped = yield (self.update_clipping, out, idx)
+            # heavyball/utils.py:3226-3232: written back into the update buffer, which has the gradient's dtype (a stochastic
+            # round into bfloat16, a plain copy otherwise)
+            out = [stochastic_round(c, rounding.noise16(philox.STREAM_UPDATE_CLIP, t, o.shape)) if o.dtype == torch.bfloat16 else c.to(o.dtype)
+                   for o, c, t in zip(out, clipped, idx)]  # fmt: skip
         update_param_(p, out, lr, self.weight_decay, self.caution, self.cautious_weight_decay, grad, rounding, idx)
 
 

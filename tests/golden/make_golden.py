@@ -352,6 +352,15 @@ def make_group_norms():
              shapes, torch.float32, 4, grad_scale=3.0)  # fmt: skip
 
 
+def make_muon_narrow_clips():
+    """Muon with an update clip under bf16 gradients: the clip writes into the bf16 update buffer (heavyball/utils.py:3226-3232)."""
+    shapes = [(8, 16), (16,), (24, 8), (4, 3, 6)]
+    run_traj("muon_updclip_l2_bf16grad", heavyball.Muon, dict(update_clipping="l2_clip_", storage_dtype="bfloat16", lr=0.02), shapes,
+             torch.bfloat16, 4)  # fmt: skip
+    run_traj("muonadamw_updclip_global_rms_bf16grad_ecc", heavyball.MuonAdamW, dict(update_clipping="global_rmsnorm_clip", ecc="bf16+8", lr=0.02),
+             shapes, torch.bfloat16, 4)  # fmt: skip
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -509,7 +518,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -530,6 +539,8 @@ if __name__ == "__main__":
         make_fp16_unfused()
     if "groupnorms" in which:
         make_group_norms()
+    if "muonnarrow" in which:
+        make_muon_narrow_clips()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:
