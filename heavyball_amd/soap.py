@@ -160,11 +160,7 @@ class SOAP(HBOptimizer):
             # one state per block (heavyball/utils.py:274-286, :1612-1623): built for the preconditioner's own state in fp32; state
             # outside it (MARS' old gradient), narrow storage and the per-block count of caution are not
             raise NotImplementedError("SOAP on the HIP kernels: split together with mars, caution, ecc, param_ecc or non-fp32 storage")
-        if mars and (ecc or storage_dtype != "float32"):
-            raise NotImplementedError("SOAP on the HIP kernels: mars together with ecc or non-fp32 storage")
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
-        if mars and self.gradient_clipping is not None:
-            raise NotImplementedError("SOAP on the HIP kernels: mars together with gradient_clipping")
         per_tensor = ("l2_clip_", "rmsnorm_clip_")
         if split and merge_dims and (self.gradient_clipping in per_tensor or self.update_clipping in per_tensor):
             raise NotImplementedError("SOAP on the HIP kernels: split together with clipping by a norm per tensor (per block in the reference)")
@@ -209,22 +205,31 @@ class SOAP(HBOptimizer):
             if group.get("mars"):
                 # heavyball/chainable.py:642-647 heads the chain and writes the corrected gradient over the gradient itself: a
                 # pass of its own leaves it in the fp32 role "_clip", which then stands for the gradient everywhere below
-                b.slab.role(K_OLD, torch.float32)
+                # mars_old_grad is stored like the moments (zero_guard with the group's storage, heavyball/chainable.py:277-301)
+                b.slab.role(K_OLD, mom_prim)
+                if mom_corr is not None:
+                    b.slab.role(K_OLD + "::ecc", mom_corr)
                 for (i, p, _), g32 in zip(items, raw[key]):
                     st = self._state0(p)
                     if K_OLD not in st:
                         st[K_OLD] = b.slab.view(K_OLD, i)
+                        if mom_corr is not None:
+                            st[K_OLD + "::ecc"] = b.slab.view(K_OLD + "::ecc", i)
                         st.setdefault("is_initialized", set()).add(5)
                 raw[key] = [g if g.data_ptr() % 16 == 0 else g.clone() for g in raw[key]]
                 lst = sorted(((i, g32) for (i, _, _), g32 in zip(items, raw[key])), key=lambda t: t[0])
-                self._mars_prologue(L, group, b, lst, torch.float32, step, *mars_weights(group), _lib.FMT_F32, K_OLD)
+                self._mars_prologue(L, group, b, lst, torch.float32, step, *mars_weights(group), mom_fmt, K_OLD)
                 raw[key] = [b.slab.view("_clip", i) for i, _, _ in items]
+                if self.gradient_clipping is not None:
+                    # the clip below rewrites the role in place; what stands for the gradient (the first factors of a tensor's
+                    # first step, heavyball/chainable.py:1235-1238, and caution's sign test) is the corrected gradient before it
+                    raw[key] = [(v.clone() if K_M not in self._state0(p) or group["caution"] else v) for v, (_, p, _) in zip(raw[key], items)]
         if self.gradient_clipping is not None:
             # heavyball/chainable.py:2696-2699: the clip acts on the update; the gradient itself still initialises the
             # factors (:1235-1238) and is what caution compares against
             work = [(b, sorted(((i, g32) for (i, _, _), g32 in zip(items, raw[key])), key=lambda t: t[0]), torch.float32)
                     for key, (b, items) in per_bucket.items()]  # fmt: skip
-            self._clip_gradients(L, group, work, step)
+            self._clip_gradients(L, group, work, step, gathered=bool(group.get("mars")))
         pending = []  # parameter updates, launched once the (optionally clipped) update of the whole group is there
         for key, (b, items) in per_bucket.items():
             b.slab.role("_update", torch.float32)

@@ -271,11 +271,11 @@ class SOAPOracle:
         updates = {i: g.clone() for i, g in enumerate(grads) if g is not None}
         if self.mars and updates:  # heavyball/chainable.py:642-647 heads the chain; the gradient becomes the corrected one
             from . import first_order as fo
-            from .rounding import HalfRounding
 
             keys = list(updates)
-            old = [self.state[k].setdefault(self.K_OLD, torch.zeros_like(grads[k])) for k in keys]
-            fo.mars_correction([updates[k] for k in keys], old, self.mars_gamma, self.betas[0], HalfRounding(), keys)
+            # zero_guard with the group's storage, like the moments (heavyball/chainable.py:277-301), in the parameter's own shape
+            old = [self._moment(self.state[k], self.K_OLD, grads[k]) for k in keys]
+            fo.mars_correction([updates[k] for k in keys], old, self.mars_gamma, self.betas[0], self.rounding.at_step(int(step)), keys)
             grads = [updates[i].clone() if i in updates else None for i in range(len(grads))]
         if self.gradient_clipping is not None and updates:  # heavyball/chainable.py:2696-2699: on the update, ahead of the transform
             from . import first_order as fo

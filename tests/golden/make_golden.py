@@ -361,6 +361,19 @@ def make_muon_narrow_clips():
              shapes, torch.bfloat16, 4)  # fmt: skip
 
 
+def make_soap_mars_combinations():
+    """SOAP with MARS ahead of narrow moments (mars_old_grad is stored like them) and ahead of a gradient clip (the factors are
+    initialised from the corrected gradient, the preconditioner sees the clipped one)."""
+    shapes = [(8, 16), (16,), (12, 6)]
+    run_traj("soap_mars_ecc", heavyball.SOAP, dict(mars=True, ecc="bf16+8", precondition_frequency=3), shapes, torch.float32, 6)
+    run_traj("soap_mars_bf16_storage_caution", heavyball.SOAP, dict(mars=True, storage_dtype="bfloat16", caution=True, precondition_frequency=3),
+             shapes, torch.float32, 6)  # fmt: skip
+    run_traj("soap_mars_clip_global_l2", heavyball.SOAP, dict(mars=True, gradient_clipping="global_l2norm_clip", precondition_frequency=3,
+                                                              mars_gamma=0.1), shapes, torch.float32, 6, grad_scale=1.0)  # fmt: skip
+    run_traj("soap_mars_clip_rms_caution", heavyball.SOAP, dict(mars=True, gradient_clipping="rmsnorm_clip_", caution=True, precondition_frequency=3),
+             shapes, torch.float32, 6, grad_scale=3.0)  # fmt: skip
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -518,7 +531,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -541,6 +554,8 @@ if __name__ == "__main__":
         make_group_norms()
     if "muonnarrow" in which:
         make_muon_narrow_clips()
+    if "soapmars" in which:
+        make_soap_mars_combinations()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:

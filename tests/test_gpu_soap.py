@@ -511,7 +511,7 @@ def test_random_soap_configurations_match_oracle(seed):
     kwargs = dict(precondition_frequency=rnd.choice([3, 4]), mars=rnd.random() < 0.3, caution=rnd.random() < 0.3,
                   weight_decay=rnd.choice([0.0, 0.01, 0.1]), max_precond_dim=rnd.choice([2048, 2048, 64, 24, 10]),
                   precondition_1d=rnd.random() < 0.3)  # fmt: skip
-    if rnd.random() < 0.25 and not kwargs["mars"]:
+    if rnd.random() < 0.25:
         kwargs["gradient_clipping"] = rnd.choice(["l2_clip_", "rmsnorm_clip_", "global_l2norm_clip", "global_rmsnorm_clip"])
     if rnd.random() < 0.25:
         kwargs["update_clipping"] = rnd.choice(["l2_clip_", "rmsnorm_clip_", "global_l2norm_clip", "global_rmsnorm_clip"])
