@@ -136,6 +136,27 @@ def step_lr_np(base_lr: float, n: int, warmup_steps: int) -> np.float32:
     return np.float32(base_lr) * np.float32(n) / np.float32(max(n, warmup_steps + 1))
 
 
+_hostloop_module = False  # False: not looked for yet; None: not built
+
+
+def hostloop():
+    """The C++ helper of the cached-plan step (csrc/hostloop.cpp, built next to libhbstep.so), or None when it has not been built:
+    the step then walks its tensors in Python, with the same checks."""
+    global _hostloop_module
+    if _hostloop_module is False:
+        import importlib.util
+        import os
+
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_hostloop.so")
+        _hostloop_module = None
+        if os.path.exists(path):
+            spec = importlib.util.spec_from_file_location("_hostloop", path)
+            mod = importlib.util.module_from_spec(spec)
+            spec.loader.exec_module(mod)
+            _hostloop_module = mod
+    return _hostloop_module
+
+
 def current_stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -181,6 +202,18 @@ class Bucket:
         if len(self.grad_tables) >= 16:
             self.grad_tables.pop(next(iter(self.grad_tables)))  # oldest first; a kernel in flight keeps its table through _last_launch
         self.grad_tables[tup] = (dev, host)
+        return dev
+
+    def grad_ptr_table_from(self, key, ptrs: torch.Tensor) -> torch.Tensor:
+        """``grad_ptr_table`` for pointers that already sit in an int64 CPU tensor; ``key``: (gradient dtype, the tensor's bytes)."""
+        hit = self.grad_tables.get(key)
+        if hit is not None:
+            return hit[0]
+        host = ptrs.clone().pin_memory() if self.device.type == "cuda" else ptrs.clone()
+        dev = host.to(self.device, non_blocking=True)
+        if len(self.grad_tables) >= 16:
+            self.grad_tables.pop(next(iter(self.grad_tables)))
+        self.grad_tables[key] = (dev, host)
         return dev
 
     def home_ptrs(self) -> List[int]:
@@ -693,7 +726,7 @@ class HBOptimizer(torch.optim.Optimizer):
 class _BucketPlan:
     """What one bucket's launch needs from step to step: the filled descriptor and the tables it points to."""
 
-    __slots__ = ("bucket", "desc", "gdt", "params", "home", "keep", "device_index")
+    __slots__ = ("bucket", "desc", "gdt", "params", "home", "keep", "device_index", "home_t", "ptrs_t", "ptrs_np")
 
 
 class _StepPlan:
@@ -823,7 +856,13 @@ class FirstOrder(HBOptimizer):
             return False
         self._note_lr(group)
         staged = []
+        helper = hostloop()
         for bp in plan.buckets:
+            if helper is not None:  # the same checks in one C++ loop over the tensors
+                if helper.collect(bp.params, bp.home_t, bp.ptrs_t, bp.gdt) != 0:
+                    return False
+                staged.append(None)
+                continue
             grads = [p.grad for p in bp.params]
             try:
                 ptrs = [g.data_ptr() for g in grads]
@@ -839,10 +878,6 @@ class FirstOrder(HBOptimizer):
             if low & 15 or [p.data_ptr() for p in bp.params] != bp.home:
                 return False
             staged.append(ptrs)
-        if self.consume_grad:
-            for bp in plan.buckets:
-                for p in bp.params:
-                    p.grad = None
         n = step_t.item() + 1
         step_t.fill_(n)
         lr = step_lr_np(base_lr, n, group["warmup_steps"])
@@ -865,7 +900,7 @@ class FirstOrder(HBOptimizer):
         current = torch.cuda.current_device()
         for bp, ptrs in zip(plan.buckets, staged):
             b, d = bp.bucket, bp.desc
-            table = b.grad_ptr_table(bp.gdt, ptrs)
+            table = b.grad_ptr_table(bp.gdt, ptrs) if ptrs is not None else b.grad_ptr_table_from((bp.gdt, bp.ptrs_np.tobytes()), bp.ptrs_t)
             d.grad_ptrs = table.data_ptr()
             d.a1, d.one_minus_a1, d.a2, d.one_minus_a2, d.eps = a1, oma1, a2, oma2, eps
             d.mars_a, d.one_minus_mars_a, d.neg_lr, d.one_minus_decay_lr = mars_a, mars_oma, neg_lr, omdl
@@ -877,6 +912,15 @@ class FirstOrder(HBOptimizer):
                     rc = L.hb_fused_step(d, current_stream_ptr(b.device))
             _lib.check(rc, "hb_fused_step")
             self._last_launch = (d, (table, bp.keep))
+        # The gradients go last: until the launches are queued nothing may free their memory, or an allocation made on the way
+        # (a new pointer table) could be handed a gradient's block and be written ahead of the kernel that reads the gradient.
+        if self.consume_grad:
+            for bp in plan.buckets:
+                if helper is not None:
+                    helper.drop_grads(bp.params)
+                    continue
+                for p in bp.params:
+                    p.grad = None
         return True
 
     #: take the un-fused form of the transform (scale_by_*, then update_param_) whenever a gradient is narrower than fp32: the
@@ -1026,6 +1070,8 @@ class FirstOrder(HBOptimizer):
                 bp = _BucketPlan()
                 bp.bucket, bp.desc, bp.gdt, bp.params, bp.home = b, d, gdt, b.params, b.home_ptrs()
                 bp.keep, bp.device_index = (chunks, offsets, numel), b.device.index
+                bp.home_t, bp.ptrs_t = torch.tensor(bp.home, dtype=torch.int64), torch.zeros(len(bp.home), dtype=torch.int64)
+                bp.ptrs_np = bp.ptrs_t.numpy()
                 plan_buckets.append(bp)
         if plannable:
             plan = _StepPlan()

@@ -624,8 +624,21 @@ PLAN_CASES = [
 ]  # fmt: skip
 
 
+@pytest.fixture(params=["cpp_loop", "python_loop"])
+def tensor_loop(request):
+    """The cached-plan step walks its tensors in the C++ helper when that is built, else in Python: both are run."""
+    from heavyball_amd import optim
+
+    assert optim.hostloop() is not None, "heavyball_amd/_hostloop.so has not been built"
+    before = optim._hostloop_module
+    if request.param == "python_loop":
+        optim._hostloop_module = None
+    yield request.param
+    optim._hostloop_module = before
+
+
 @pytest.mark.parametrize("case", PLAN_CASES, ids=[c[0] for c in PLAN_CASES])
-def test_cached_plan_steps_equal_the_general_path(case):
+def test_cached_plan_steps_equal_the_general_path(case, tensor_loop):
     """``FirstOrder._fast_step`` replays the launches of the step before with new scalars and gradient pointers.  Two optimizers
     on the same inputs, one with the cached plan switched off, stay bit-identical through ordinary steps and through everything
     that must send a step back to the general path: a missing gradient, a changed learning rate and betas (which the plan reads

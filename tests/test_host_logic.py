@@ -204,3 +204,40 @@ def test_corr_over_smax_newton_step_is_correctly_rounded_for_every_correction():
         mid = (q.astype(np.float64) + np.nextafter(q, np.where(exact > q, np.float32(np.inf), np.float32(-np.inf))).astype(np.float64)) / 2
         assert (np.abs(exact - mid) > 4 * np.spacing(np.abs(exact))).all()
         assert np.array_equal(q.view(np.uint32), want.view(np.uint32)), smax
+
+
+def test_cpp_tensor_loop_checks_what_the_python_loop_checks():
+    """csrc/hostloop.cpp on CPU tensors: the gradients' addresses when every tensor passes, and the reason code for each thing that
+    sends a step back to the general path (a missing gradient, another dtype, a strided gradient, a misaligned one, a parameter
+    whose data moved); ``drop_grads`` leaves every gradient None."""
+    helper = optim.hostloop()
+    assert helper is not None, "heavyball_amd/_hostloop.so has not been built (make -C heavyball_amd/csrc)"
+    ps = [torch.nn.Parameter(torch.randn(8, 16)) for _ in range(5)]
+    for p in ps:
+        p.grad_dtype = None
+    gs = [torch.randn(8, 16).bfloat16() for _ in ps]
+
+    def arm():
+        for p, g in zip(ps, gs):
+            p.grad = g
+
+    arm()
+    home = torch.tensor([p.data_ptr() for p in ps], dtype=torch.int64)
+    out = torch.zeros(len(ps), dtype=torch.int64)
+    assert helper.collect(ps, home, out, torch.bfloat16) == 0
+    assert out.tolist() == [g.data_ptr() for g in gs]
+    assert helper.collect(ps, home, out, torch.float32) == 2
+    ps[3].grad = None
+    assert helper.collect(ps, home, out, torch.bfloat16) == 1
+    arm()
+    ps[1].grad = torch.randn(16, 8).bfloat16().t()  # same shape, column-major
+    assert helper.collect(ps, home, out, torch.bfloat16) == 3
+    arm()
+    ps[2].grad = torch.randn(8 * 16 + 1).bfloat16()[1:].view(8, 16)  # two bytes off a 16-byte boundary
+    assert ps[2].grad.data_ptr() % 16 and helper.collect(ps, home, out, torch.bfloat16) == 4
+    arm()
+    ps[4].data = ps[4].data.clone()
+    assert helper.collect(ps, home, out, torch.bfloat16) == 5
+    assert helper.collect(ps, home[:3], out, torch.bfloat16) == 6  # tables of another length
+    helper.drop_grads(ps)
+    assert all(p.grad is None for p in ps)
