@@ -174,13 +174,15 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
           const float t1 = g[j] * a.omamars, t2 = bf16_to_f32(ho) * a.amars;
           gs = t1 + t2;  // the corrected gradient before its rounding, from the primary of old_grad
           // what the correction of old_grad and the fp32 roundings can move
-          const float eo = __builtin_fabsf(t2) * k_ulp + (__builtin_fabsf(t1) + __builtin_fabsf(t2)) * 0x1p-22f + c_o;
+          // (the bounds are not part of the reference's arithmetic: fused multiply-adds, whose single rounding the 1.01 covers)
+          const float eo = __builtin_fmaf(__builtin_fabsf(t2), k_ulp, __builtin_fmaf(__builtin_fabsf(t1) + __builtin_fabsf(t2), 0x1p-22f, c_o));
           sure = __builtin_fabsf(gs) > eo;  // its sign is settled (the stochastic rounding to bf16 keeps the sign)
-          dg = eo + (__builtin_fabsf(gs) + eo) * 0x1p-7f + 1e-39f;  // ... and its value to within one bf16 ulp more
+          dg = __builtin_fmaf(__builtin_fabsf(gs) + eo, 0x1p-7f, eo) + 1e-39f;  // ... and its value to within one bf16 ulp more
         }
         const float s1 = mp * a.oma1, s2 = gs * a.a1;
         const float mn = s1 + s2;
-        const float em = __builtin_fabsf(s1) * k_ulp + k_a1 * dg + (__builtin_fabsf(s1) + __builtin_fabsf(s2)) * 0x1p-21f + c_m;
+        const float em = __builtin_fmaf(__builtin_fabsf(s1), k_ulp,
+                                        __builtin_fmaf(k_a1, dg, __builtin_fmaf(__builtin_fabsf(s1) + __builtin_fabsf(s2), 0x1p-21f, c_m)));
         sure = sure && __builtin_fabsf(mn) > em;  // NaN compares false: the exact route decides
         const bool inside = FULL || e + j < valid;
         if (inside && !sure) undecided |= 1u << j;
