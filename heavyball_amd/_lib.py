@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("HBSTEP_LIB") or os.path.join(_HERE, "libhbstep.so")
 
 # include/hbstep.h
-ABI_VERSION = 8  # HB_ABI_VERSION this binding was written against
+ABI_VERSION = 9  # HB_ABI_VERSION this binding was written against
 FMT_F32, FMT_BF16, FMT_F16, FMT_ECC_BF16_8, FMT_ECC_BF16_16, FMT_ECC_F16_8, FMT_ECC_F16_16 = range(7)
 ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD, FLAG_MARS_ONLY = 1, 2, 4, 8, 16, 32, 64, 128
@@ -21,7 +21,8 @@ RNG_HALF, RNG_PHILOX = 0, 1
 STREAM_MARS_SR, STREAM_PARAM, STREAM_EXP_AVG, STREAM_EXP_AVG_SQ, STREAM_OLD_GRAD, STREAM_INIT_PARAM, STREAM_NS_INPUT = range(7)
 STREAM_CLIP, STREAM_EXP_AVG_SLOW, STREAM_UPDATE, STREAM_SOAP_ROTATE, STREAM_UPDATE_CLIP = 8, 9, 10, 11, 12
 NS_LEGACY, NS_BF16_UPDATE = 1, 2
-NOALLOC_MAX_TENSORS = 65536  # HB_NOALLOC_MAX_TENSORS
+NOALLOC_MAX_TENSORS = 8192  # HB_NOALLOC_MAX_TENSORS
+CAUTION_SLOTS = 32  # HB_CAUTION_SLOTS: counters per tensor in HbStepDesc.caution_count
 GEMM_ACCUMULATE, GEMM_SYMMETRIC = 1, 2
 MOM_NESTEROV_EMA, MOM_EMA, MOM_HEAVYBALL, MOM_NESTEROV_HEAVYBALL = range(4)
 

@@ -31,6 +31,7 @@ extern template StepKernel pick_algo<HB_ALGO_NADAM>(bool, int, int, int, int);
 // against the gradient.  COUNT = 1 only counts masked elements.
 constexpr int kUThreads = 256;                           // update_param_kernel: one workgroup per chunk,
 constexpr int kUGroups = HB_CHUNK / (kUThreads * 8);     // kUGroups octets per lane
+static_assert(kUThreads == kThreads, "add_masked sizes its LDS words for kThreads lanes");
 template <int CAUTION, int PF>
 __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs a) {
   const int pf = PF == kDyn ? a.pf : PF;
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs 
     const int64_t g0 = g_slab ? flat0 : local0;
     float scale = 1.0f;
     if (CAUTION == kCautionApply) {
-      const int64_t kept = n - (int64_t)a.counts[t];
+      const int64_t kept = n - masked_of(a.counts, t);
       scale = (1.0f / (float)(kept < 1 ? 1 : kept)) * (float)n;  // reciprocal(kept) * numel, as in the fused step
     }
     uint32_t masked = 0;
@@ -89,10 +90,7 @@ __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs 
         raw_put<PF>(pf, p, rn, a.param, a.param_corr, idx);
       }
     }
-    if (kCount) {
-      masked = wave_sum(masked);
-      if ((threadIdx.x & (kWave - 1)) == 0 && masked) atomicAdd(&a.counts[t], masked);
-    }
+    if (kCount) add_masked(a.counts, t, (int)(c & (HB_CAUTION_SLOTS - 1)), masked);
   }
 }
 
@@ -225,7 +223,7 @@ static int run_fused_step(const HbStepDesc* d, StepArgs& a, uint32_t* counts, hi
   };
   bool ok;
   if (caution) {
-    zero_u32_kernel<<<(d->n_tensors + 255) / 256, 256, 0, stream>>>(counts, d->n_tensors);
+    zero_u32_kernel<<<(d->n_tensors * HB_CAUTION_SLOTS + 255) / 256, 256, 0, stream>>>(counts, d->n_tensors * HB_CAUTION_SLOTS);
     ok = launch(kCautionCount) && launch(kCautionApply);
   } else {
     ok = launch(kNoCaution);
@@ -236,7 +234,7 @@ static int run_fused_step(const HbStepDesc* d, StepArgs& a, uint32_t* counts, hi
 
 // Scratch of hb_fused_step_noalloc: the caution counters live in the library's own device memory.  Every device the
 // library runs on holds its own copy of this array at its own address, for the life of the process.
-static __device__ __align__(256) uint32_t scratch[HB_NOALLOC_MAX_TENSORS];
+static __device__ __align__(256) uint32_t scratch[HB_NOALLOC_MAX_TENSORS * HB_CAUTION_SLOTS];
 
 constexpr int kMaxDevices = 64;
 static std::atomic<uint32_t*> g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device, resolved once
@@ -290,7 +288,7 @@ extern "C" int hb_update_param(const HbStepDesc* d, void* stream_) {
   const int grid = persistent_grid(d->n_chunks);
   if (grid <= 0) return set_error(HB_ELAUNCH, "could not query the device");
   if (caution) {
-    zero_u32_kernel<<<(d->n_tensors + 255) / 256, 256, 0, stream>>>(d->caution_count, d->n_tensors);
+    zero_u32_kernel<<<(d->n_tensors * HB_CAUTION_SLOTS + 255) / 256, 256, 0, stream>>>(d->caution_count, d->n_tensors * HB_CAUTION_SLOTS);
     update_param_kernel<kCautionCount, kDyn><<<grid, kUThreads, 0, stream>>>(a);
     update_param_kernel<kCautionApply, kDyn><<<grid, kUThreads, 0, stream>>>(a);
   } else if (a.pf == HB_FMT_F32) {

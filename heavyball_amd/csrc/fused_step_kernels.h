@@ -72,11 +72,39 @@ __device__ __forceinline__ void for_each_index(F&& f, std::integer_sequence<int,
   (f(std::integral_constant<int, K>{}), ...);
 }
 
+// The masked elements a workgroup counted go into one of the tensor's HB_CAUTION_SLOTS counters: one addition per workgroup
+// (wavefront shuffles, then four words of LDS), and neighbouring workgroups add into different words.  Additions to one
+// address queue up in the L2 (about 200 M a second measured): with one counter per tensor and one addition per wavefront
+// the count pass of a training-like state, where every wavefront has masked elements, spent five times its streaming time there.
+__device__ __forceinline__ void add_masked(uint32_t* counts, int t, int slot, uint32_t masked) {
+  __shared__ uint32_t per_wave[kThreads / kWave];
+  masked = wave_sum(masked);
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) per_wave[wave] = masked;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t total = 0;
+#pragma unroll
+    for (int i = 0; i < kThreads / kWave; ++i) total += per_wave[i];
+    if (total) atomicAdd(&counts[(size_t)t * HB_CAUTION_SLOTS + slot], total);
+  }
+  __syncthreads();  // the words are reused by the workgroup's next work unit
+}
+
+// the masked elements of tensor t: the sum of its counters
+__device__ __forceinline__ int64_t masked_of(const uint32_t* counts, int t) {
+  const uint32_t* c = counts + (size_t)t * HB_CAUTION_SLOTS;
+  uint32_t total = 0;  // a tensor has fewer than 2^32 elements
+#pragma unroll
+  for (int i = 0; i < HB_CAUTION_SLOTS; ++i) total += c[i];
+  return (int64_t)total;
+}
+
 // One work unit.  FULL = every lane's elements are inside the tensor (the common case): no bounds tests at all.
 template <int ALGO, bool MARS, int CAUTION, int PF, int GF, int SF, bool FULL, class GEO>
 __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, const int gf, const int sf, const int t, const int valid,
                                            const int64_t flat0, const char* gbase, const int64_t g0, const bool g_slab, const float scale,
-                                           const float gw, const float ew) {
+                                           const float gw, const float ew, const int slot) {
   constexpr int kE = GEO::E, kGroups = GEO::G;
   constexpr bool kCount = CAUTION == kCautionCount;
   constexpr bool kAdopt = ALGO == HB_ALGO_ADOPT, kMix = ALGO == HB_ALGO_ADEMAMIX, kNadam = ALGO == HB_ALGO_NADAM;
@@ -193,6 +221,9 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
       // three quarters of the wavefronts (64 lanes of 8 elements), so it has to cost a wavefront little: one quartet's random
       // numbers and the flagged elements alone, not the whole group with every lane but one idle.
       if (undecided) {
+        // both correction words first, so that the flagged elements wait for memory once and not one after the other
+        ld_slab<kE>(a.m_corr + idx, rm[k].c);
+        if (MARS) ld_slab<kE>(a.og_corr + idx, ro[k].c);
 #pragma unroll
         for (int q = 0; q < kE / 4; ++q) {
           if (!(undecided & (0xFu << (4 * q)))) continue;
@@ -203,11 +234,11 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
             const int j = 4 * q + jj;
             if (!((undecided >> j) & 1u)) continue;
             const uint32_t hm = (rm[k].a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
-            const float mx = ecc_decode<true, true>(hm, (int)ld_as<int8_t>(a.m_corr + idx + j));
+            const float mx = ecc_decode<true, true>(hm, (int)(int8_t)(rm[k].c[j >> 2] >> ((j & 3) * 8)));
             float gc = g[j];
             if (MARS) {
               const uint32_t ho = (ro[k].a[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
-              const float ox = ecc_decode<true, true>(ho, (int)ld_as<int8_t>(a.og_corr + idx + j));
+              const float ox = ecc_decode<true, true>(ho, (int)(int8_t)(ro[k].c[j >> 2] >> ((j & 3) * 8)));
               gc = g[j] * a.omamars + ox * a.amars;  // heavyball/utils.py:1048, then its rounding to the gradient's bf16
               gc = bf16_to_f32(sr_bf16(gc, (r.w[jj >> 1] >> ((jj & 1) * 16)) & 0xFFFFu));  // word and half of HB_STREAM_MARS_SR
             }
@@ -359,10 +390,7 @@ __device__ __forceinline__ void step_chunk(const StepArgs& a, const int pf, cons
   };
   for_each_index(group, std::make_integer_sequence<int, kGroups>{});
 
-  if (kCount) {
-    masked = wave_sum(masked);
-    if ((threadIdx.x & (kWave - 1)) == 0 && masked) atomicAdd(&a.counts[t], masked);
-  }
+  if (kCount) add_masked(a.counts, t, slot, masked);
 }
 
 #ifndef HB_COUNT_WAVES  // wavefronts per SIMD the compiler must leave room for (its register budget) in the count pass ...
@@ -392,7 +420,7 @@ __global__ __launch_bounds__(kThreads, CAUTION == kCautionCount ? HB_COUNT_WAVES
     const int64_t g0 = g_slab ? flat0 : local0;
     float scale = 1.0f;
     if (CAUTION == kCautionApply) {
-      const int64_t kept = n - (int64_t)a.counts[t];
+      const int64_t kept = n - masked_of(a.counts, t);
       // heavyball/utils.py:3656: `numel / kept_tensor` is Tensor.__rtruediv__, i.e. reciprocal(kept) * numel in fp32
       scale = (1.0f / (float)(kept < 1 ? 1 : kept)) * (float)n;
     }
@@ -401,8 +429,9 @@ __global__ __launch_bounds__(kThreads, CAUTION == kCautionCount ? HB_COUNT_WAVES
       gw = a.tscal[2 * t];
       ew = a.tscal[2 * t + 1];
     }
-    if (valid == kWork) step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, true, GEO>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
-    else step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, false, GEO>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew);
+    const int slot = (int)(w & (HB_CAUTION_SLOTS - 1));
+    if (valid == kWork) step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, true, GEO>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew, slot);
+    else step_chunk<ALGO, MARS, CAUTION, PF, GF, SF, false, GEO>(a, pf, gf, sf, t, valid, flat0, gbase, g0, g_slab, scale, gw, ew, slot);
   }
 }
 

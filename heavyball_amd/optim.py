@@ -184,7 +184,7 @@ class Bucket:
 
     def caution_scratch(self) -> torch.Tensor:
         if self.counts is None:
-            self.counts = torch.zeros(len(self.params), dtype=torch.int32, device=self.device)
+            self.counts = torch.zeros(len(self.params) * _lib.CAUTION_SLOTS, dtype=torch.int32, device=self.device)
         return self.counts
 
     def grad_ptr_table(self, key, ptrs: List[int]) -> torch.Tensor:

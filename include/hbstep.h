@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 8
+#define HB_ABI_VERSION 9
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -117,6 +117,9 @@ enum {
  * per tensor (`grad_ptrs`, device array, each 16-byte aligned); exactly one of the two is non-null.
  * `chunks[c] = {tensor, chunk index inside the tensor}` lists the work; tensors without a gradient are left out.
  */
+/* counters per tensor in HbStepDesc.caution_count */
+#define HB_CAUTION_SLOTS 32
+
 typedef struct HbStepDesc {
   void* param;
   void* param_corr; /* ECC formats only */
@@ -131,7 +134,9 @@ typedef struct HbStepDesc {
   const int64_t* offsets;  /* [n_tensors]   */
   const int64_t* numel;    /* [n_tensors]   */
   const int32_t* chunks;   /* [n_chunks][2] */
-  uint32_t* caution_count; /* [n_tensors] scratch, HB_FLAG_CAUTION only; the call zeroes and fills it */
+  uint32_t* caution_count; /* [n_tensors][HB_CAUTION_SLOTS] scratch, HB_FLAG_CAUTION only; the call zeroes and fills it: the
+                              masked elements of tensor t are the sum of its slots (workgroups add into the slot their work
+                              unit's index picks, so that the additions of one tensor do not queue up on one address) */
   int64_t n_chunks;
   int32_t n_tensors;
   int32_t algo;
@@ -170,11 +175,11 @@ int hb_fused_step(const HbStepDesc* desc, void* stream);
 /* hb_fused_step for callers that cannot allocate device memory or hand over a scratch buffer: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
  * descriptor and results as hb_fused_step, except that `caution_count` is ignored (it may be NULL): the per-tensor
- * caution counters live in a device array inside the library (4 * HB_NOALLOC_MAX_TENSORS bytes on every GPU the
- * library runs on, held until the process ends).  More than HB_NOALLOC_MAX_TENSORS tensors: HB_EINVAL.  The call
+ * caution counters live in a device array inside the library (4 * HB_CAUTION_SLOTS * HB_NOALLOC_MAX_TENSORS bytes = 1 MiB on
+ * every GPU the library runs on, held until the process ends).  More than HB_NOALLOC_MAX_TENSORS tensors: HB_EINVAL.  The call
  * allocates and frees nothing and clears the counters it uses with a fill kernel.  Every call on one GPU shares that
  * GPU's array, so two calls with HB_FLAG_CAUTION that overlap on one GPU (different streams or threads) race. */
-#define HB_NOALLOC_MAX_TENSORS 65536
+#define HB_NOALLOC_MAX_TENSORS 8192
 int hb_fused_step_noalloc(const HbStepDesc* desc, void* stream);
 
 /* chain()'s non-fused tail, update_param_ (heavyball/utils.py:2393-2406): p <- p*(1 - decay*lr) + u*(-lr) on a slab,

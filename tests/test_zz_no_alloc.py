@@ -43,7 +43,8 @@ class Roles:
         self.og, self.og_corr = role(sf, 1e-3)
         self.off_dev = torch.from_numpy(self.offsets.copy()).to(dev)
         self.numel_dev = torch.tensor(self.numels, dtype=torch.int64, device=dev)
-        self.counts = torch.full((len(self.numels),), 12345, dtype=torch.int32, device=dev)  # hb_fused_step's caller-owned scratch
+        # hb_fused_step's caller-owned scratch
+        self.counts = torch.full((len(self.numels) * _lib.CAUTION_SLOTS,), 12345, dtype=torch.int32, device=dev)
 
     def buffers(self):
         return {k: getattr(self, k) for k in ("param", "param_corr", "m", "m_corr", "v", "v_corr", "og", "og_corr") if getattr(self, k) is not None}
@@ -90,7 +91,7 @@ def test_noalloc_entry_matches_fused_step_on_two_calls(case):
         _lib.check(L.hb_fused_step(ctypes.byref(d_ref), stream), "hb_fused_step")
         _lib.check(L.hb_fused_step_noalloc(ctypes.byref(d_new), stream), "hb_fused_step_noalloc")
         torch.cuda.synchronize()
-        masked = ref.counts.cpu()
+        masked = ref.counts.cpu().view(-1, _lib.CAUTION_SLOTS).sum(1)
         assert all(int(masked[i]) > 0 for i in active), "the case must exercise the counters"
         for name, want in ref.buffers().items():
             got = new.buffers()[name]
@@ -107,6 +108,6 @@ def test_noalloc_entry_rejects_more_tensors_than_its_scratch_holds():
     before = r.param.clone()
     d.n_tensors = _lib.NOALLOC_MAX_TENSORS + 1
     assert L.hb_fused_step_noalloc(ctypes.byref(d), torch.cuda.current_stream(dev).cuda_stream) == -1
-    assert b"at most 65536" in L.hb_last_error()
+    assert b"at most 8192" in L.hb_last_error()
     torch.cuda.synchronize()
     assert torch.equal(r.param, before)  # nothing was launched
