@@ -29,22 +29,29 @@ extern template StepKernel pick_algo<HB_ALGO_NADAM>(bool, int, int, int, int);
 
 // chain()'s non-fused tail (heavyball/utils.py:2393-2406): the update is an fp32 slab (in a.m), optional caution
 // against the gradient.  COUNT = 1 only counts masked elements.
-constexpr int kUThreads = 256;                           // update_param_kernel: one workgroup per chunk,
-constexpr int kUGroups = HB_CHUNK / (kUThreads * 8);     // kUGroups octets per lane
+constexpr int kUThreads = 256;                 // update_param_kernel: a lane owns kUE consecutive elements, a workgroup kUWork,
+#ifndef HB_UPD_E
+#define HB_UPD_E 4
+#endif
+constexpr int kUE = HB_UPD_E;                   // and a chunk is kUSub such work units (short runs per lane: see muon.hip)
+constexpr int kUWork = kUThreads * kUE;
+constexpr int kUSub = HB_CHUNK / kUWork;
 static_assert(kUThreads == kThreads, "add_masked sizes its LDS words for kThreads lanes");
+static_assert(kUSub * kUWork == HB_CHUNK && (kUE == 4 || kUE == 8), "a chunk is a whole number of work units");
 template <int CAUTION, int PF>
 __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs a) {
   const int pf = PF == kDyn ? a.pf : PF;
   constexpr bool kCount = CAUTION == kCautionCount;
   const bool cautious_wd = (a.flags & HB_FLAG_CAUTIOUS_WD) != 0;
-  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
-    const int2 ent = a.chunks[c];
+  for (int64_t w = blockIdx.x; w < a.n_chunks * kUSub; w += gridDim.x) {
+    const int2 ent = a.chunks[w / kUSub];
     const int t = ent.x;
     const int64_t off = a.offsets[t];
     const int64_t n = a.numel[t];
-    const int64_t local0 = (int64_t)ent.y * HB_CHUNK;
+    const int64_t local0 = (int64_t)ent.y * HB_CHUNK + (int64_t)(w % kUSub) * kUWork;
     const int64_t rem = n - local0;
-    const int valid = rem < HB_CHUNK ? (int)rem : HB_CHUNK;
+    if (rem <= 0) continue;  // a work unit behind the end of the tensor's last chunk
+    const int valid = rem < kUWork ? (int)rem : kUWork;
     const int64_t flat0 = off + local0;
     const bool g_slab = a.grad_ptrs == nullptr;
     const char* gbase = CAUTION != kNoCaution ? (g_slab ? a.grad : a.grad_ptrs[t]) : nullptr;
@@ -55,25 +62,23 @@ __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs 
       scale = (1.0f / (float)(kept < 1 ? 1 : kept)) * (float)n;  // reciprocal(kept) * numel, as in the fused step
     }
     uint32_t masked = 0;
-#pragma unroll
-    for (int k = 0; k < kUGroups; ++k) {
-      const int e = k * (kUThreads * 8) + threadIdx.x * 8;
-      if (e >= valid) continue;
+    const int e = threadIdx.x * kUE;
+    if (e < valid) {
       const int64_t idx = flat0 + e;
-      Raw ru, rp;
-      float u[8], p[8], g[8];
+      RawT<kUE> ru, rp;
+      float u[kUE], p[kUE], g[kUE];
       if (a.sf == HB_FMT_BF16) raw_load<HB_FMT_BF16>(ru, HB_FMT_BF16, a.m, nullptr, idx);  // the update as a bf16 slab
       else raw_load<HB_FMT_F32>(ru, HB_FMT_F32, a.m, nullptr, idx);
       if (!kCount) raw_load<PF>(rp, pf, a.param, a.param_corr, idx);
       if (CAUTION != kNoCaution) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) g[j] = e + j < valid ? load_elem(gbase, a.gf, g0 + e + j) : 0.0f;
+        for (int j = 0; j < kUE; ++j) g[j] = e + j < valid ? load_elem(gbase, a.gf, g0 + e + j) : 0.0f;
       }
       if (a.sf == HB_FMT_BF16) raw_decode<HB_FMT_BF16>(ru, HB_FMT_BF16, u);
       else raw_decode<HB_FMT_F32>(ru, HB_FMT_F32, u);
       if (!kCount) raw_decode<PF>(rp, pf, p);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kUE; ++j) {
         if (CAUTION != kNoCaution) {
           const bool mk = ((f2u(g[j]) ^ f2u(u[j])) >> 31) != 0;
           if (kCount) masked += (mk && e + j < valid) ? 1u : 0u;
@@ -86,11 +91,11 @@ __global__ __launch_bounds__(kUThreads) void update_param_kernel(const StepArgs 
         }
       }
       if (!kCount) {
-        Rand8 rn = pf != HB_FMT_F32 ? a.rng.octet(idx, HB_STREAM_PARAM) : Rand8{{0, 0, 0, 0}};
+        const Noise<kUE> rn = pf != HB_FMT_F32 ? a.rng.noise<kUE>(idx, HB_STREAM_PARAM) : Noise<kUE>{};
         raw_put<PF>(pf, p, rn, a.param, a.param_corr, idx);
       }
     }
-    if (kCount) add_masked(a.counts, t, (int)(c & (HB_CAUTION_SLOTS - 1)), masked);
+    if (kCount) add_masked(a.counts, t, (int)(w & (HB_CAUTION_SLOTS - 1)), masked);
   }
 }
 
@@ -285,7 +290,7 @@ extern "C" int hb_update_param(const HbStepDesc* d, void* stream_) {
   if (d->n_chunks == 0) return HB_OK;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   const bool caution = (d->flags & HB_FLAG_CAUTION) != 0;
-  const int grid = persistent_grid(d->n_chunks);
+  const int grid = persistent_grid(d->n_chunks * kUSub);
   if (grid <= 0) return set_error(HB_ELAUNCH, "could not query the device");
   if (caution) {
     zero_u32_kernel<<<(d->n_tensors * HB_CAUTION_SLOTS + 255) / 256, 256, 0, stream>>>(d->caution_count, d->n_tensors * HB_CAUTION_SLOTS);
