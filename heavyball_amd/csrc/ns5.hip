@@ -21,6 +21,8 @@
 // conflict free.  Fragment reads and loads are issued one per MFMA, in the shadow of the matrix instruction; one
 // barrier per K-tile.
 #include <algorithm>
+#include <cstring>
+#include <functional>
 #include <vector>
 
 #include "hb_device.h"
@@ -34,8 +36,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 enum { kModeS = 0, kModeY2 = 1, kModeX = 2, kModeFinal = 3, kModePartial = 4 };  // kModePartial: raw fp32 product of one K chunk
 
-// One matrix of a grouped launch.  A launch multiplies up to kMaxGroup independent matrices: workgroup ids
-// [tile_begin, tile_begin + 8 * ceil(n_tiles / 8)) belong to this one.
+// One entry of a grouped launch: a run of consecutive tiles of one matrix, on one XCD (see locate_tile).  A launch multiplies
+// any number of independent matrices.
 struct Problem {
   const uint16_t* A;  // [M, K], row stride lda
   const uint16_t* B;  // [N, K], row stride ldb
@@ -47,16 +49,17 @@ struct Problem {
   float scale;                       // ModeFinal: post-scale
   float mul_c, diag;                 // ModeS: c and b; ModeY2: diag = a (per matrix: one launch may mix coefficient schedules)
   int tiles_m, tiles_n;              // tile grid of C
-  int tile_begin;                    // first workgroup id (a multiple of 8)
-  int n_tiles;                       // tiles computed: the upper triangle of the grid in the symmetric modes, else all
+  int pos_begin;                     // where this run starts in the tile list of its XCD
+  int t0, n_run;                     // the run: tiles t0 .. t0 + n_run - 1 of the matrix' tile list
+  int round_out;  // ModeFinal: the reference's update buffer is bf16, so the scaled result is rounded to bf16 (to nearest)
 };
-constexpr int kMaxGroup = 28;
-struct GroupArgs {
-  Problem p[kMaxGroup];
-  int n_problems;
-  int round_out;      // ModeFinal: the reference's update buffer is bf16, so the scaled result is rounded to bf16 (to nearest)
+static_assert(sizeof(Problem) % 16 == 0, "tables of problems are moved in 16-byte pieces");
+// A table: this header, then the entries of XCD 0, of XCD 1, ...; entries [first[x], first[x + 1]) are XCD x's, in list order
+struct TableHeader {
+  int first[9];
+  int pad_[7];
 };
-static_assert(sizeof(GroupArgs) <= 4096, "the group travels as a kernel argument");
+static_assert(sizeof(TableHeader) == 64, "the entries start 16-byte aligned");
 
 // LDS tile layout: one row of BK bf16 (BK*2 bytes) per matrix row, its 16-byte chunks XOR-swizzled so that the 128-bit
 // fragment reads are conflict free.  A wavefront's ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle and
@@ -72,26 +75,41 @@ __device__ __forceinline__ uint32_t lds_off(int row, int chunk) {
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-// Workgroup -> (matrix, tile).  Workgroup ids go round-robin over the 8 XCDs (each with its own L2), so XCD x runs
-// the ids congruent to x.  Every matrix starts at an id that is a multiple of 8 and hands XCD x the x-th eighth of its
-// tile list, a contiguous run: consecutive tiles share an operand panel, so the panels an XCD touches at a time stay
-// few, while every XCD gets the same mix of long and short tiles (matrices are listed longest K first).
-// In the symmetric modes the tile list is the upper triangle of the grid, row by row.
+// Workgroup -> (matrix, tile).  Workgroup ids go round-robin over the 8 XCDs (each with its own L2), so XCD x runs the ids
+// congruent to x, in order: id b is position b / 8 of XCD (b % 8)'s tile list.  The host fills these lists (gemm_stage):
+//   * a matrix with many tiles hands XCD x the x-th eighth of its tile list, a contiguous run: consecutive tiles share an
+//     operand panel, so the panels an XCD touches at a time stay few;
+//   * a matrix with few tiles (the 128-wide class) goes to ONE XCD as a whole: its tiles start together and walk K in step, so
+//     each panel comes into that XCD's L2 once and serves every tile that needs it.  Dealt out in eighths, every XCD fetches
+//     nearly every panel (a 6 x 6 triangle touches 5 of its 6 panels per XCD) and the products of a GPT-2-sized bucket run at
+//     the pace of the memory-side traffic instead of the matrix cores';
+//   * every list is ordered longest K first (the hardware starts workgroups in id order, so the long tiles start first and
+//     the short ones fill in behind them), and the lists carry equal work (longest-processing-time assignment).
+// In the symmetric modes the tile list of a matrix is the upper triangle of the grid, in strips.
 //
-// The group is read through the kernel-argument segment pointer (constant address space): indexing the by-value
-// argument with a run-time index would make the compiler copy it to scratch memory.
-typedef const __attribute__((address_space(4))) GroupArgs* group_ptr_t;
+// The lists live in a table in device memory, written before the first product of a call (a bucket of a GPT-2-sized model
+// has more matrices than a kernel argument holds, and one launch over all of them balances where two launches each end in a
+// half-empty round).  The table is read-only while a product runs, so it is read through the constant address space, i.e.
+// with scalar loads; the entry of a workgroup is found by bisection.
+typedef const __attribute__((address_space(4))) Problem* table_ptr_t;
+typedef const __attribute__((address_space(4))) TableHeader* header_ptr_t;
 
 template <bool SYMMETRIC>
-__device__ __forceinline__ bool locate_tile(group_ptr_t g, int bid, int& pi, int& bi, int& bj) {
-  pi = 0;
-  const int n_problems = g->n_problems;
-  while (pi + 1 < n_problems && bid >= g->p[pi + 1].tile_begin) ++pi;
-  const int local = bid - g->p[pi].tile_begin;
-  const int n_tiles = g->p[pi].n_tiles;
-  const int per = (n_tiles + 7) >> 3;
-  const int t = (local & 7) * per + (local >> 3);
-  if (t >= n_tiles) return false;
+__device__ __forceinline__ bool locate_tile(const void* table, int bid, table_ptr_t& g, int& pi, int& bi, int& bj) {
+  const header_ptr_t hdr = (header_ptr_t) reinterpret_cast<uintptr_t>(table);
+  g = (table_ptr_t)(reinterpret_cast<uintptr_t>(table) + sizeof(TableHeader));
+  const int x = bid & 7, pos = bid >> 3;
+  int lo = hdr->first[x], hi = hdr->first[x + 1] - 1;
+  if (lo > hi) return false;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (pos >= g[mid].pos_begin) lo = mid;
+    else hi = mid - 1;
+  }
+  pi = lo;
+  const int local = pos - g[pi].pos_begin;
+  if (local >= g[pi].n_run) return false;  // past the end of a list that is shorter than the longest one
+  const int t = g[pi].t0 + local;
 #ifndef HB_NS_STRIP
 #define HB_NS_STRIP 4
 #endif
@@ -99,7 +117,7 @@ __device__ __forceinline__ bool locate_tile(group_ptr_t g, int bid, int& pi, int
   if (SYMMETRIC) {
     // upper triangle in strips of kStrip tile rows; inside a strip column by column (the first columns of a strip are
     // cut by the diagonal), so that a run of consecutive tiles is a compact block here too
-    const int T = g->p[pi].tiles_n;
+    const int T = g[pi].tiles_n;
     int first = 0, rem = t;
     for (;;) {
       const int h = T - first < kStrip ? T - first : kStrip;
@@ -120,7 +138,7 @@ __device__ __forceinline__ bool locate_tile(group_ptr_t g, int bid, int& pi, int
   } else {
     // strips of kStrip tile rows, walked column by column: a run of consecutive tiles then covers a compact block
     // (kStrip rows x run/kStrip columns) and shares few operand panels
-    const int tiles_m = g->p[pi].tiles_m, tiles_n = g->p[pi].tiles_n;
+    const int tiles_m = g[pi].tiles_m, tiles_n = g[pi].tiles_n;
     const int strip = t / (kStrip * tiles_n), in_strip = t % (kStrip * tiles_n);
     const int first = strip * kStrip;
     const int height = tiles_m - first < kStrip ? tiles_m - first : kStrip;
@@ -162,7 +180,7 @@ __device__ __forceinline__ void wait_vmcnt(int n) {  // s_waitcnt vmcnt(n) only 
 // The epilogue of both product kernels.  Accumulator register r of tile (i, j) of a wavefront holds row
 // (r/4)*8 + (lane/32)*4 + r%4, column lane%32 of the 32 x 32 block.
 template <int MODE, int TM, int TN, int WTM, int WTN>
-__device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Problem& g, const int round_out, const int row0, const int col0,
+__device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Problem& g, const int row0, const int col0,
                                             const int wm, const int wn, const int lane, const int bi, const int bj) {
   constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
   const int erow = (lane >> 5) * 4, lcol = lane & 31;
@@ -219,7 +237,7 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
               o[r] = acc[i][j][rb4 * 4 + r];  // one K chunk of a split product: summed and rounded by ns_split_reduce_kernel
             } else {
               o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
-              if (round_out) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
+              if (g.round_out) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
             }
           }
           if (g.f_transposed) {
@@ -258,7 +276,7 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
 }
 
 template <int BM, int BN, int BK, int STAGES, int WGM, int WGN, int MODE>
-__global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs grp) {
+__global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const void* table) {
   constexpr int NW = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -272,15 +290,15 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
   static_assert(STAGES >= 2 && STAGES <= 4 && (STAGES == 2 || LOADS % 4 == 0) && 2 * LOADS <= 32 && KS % 2 == 0 && TM + TN <= 15, "pipeline bookkeeping");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
+  constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2 || MODE == kModePartial;  // the tile list is the upper triangle
   int pi, bi, bj;
-  const group_ptr_t ka = (group_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();  // the group is the first (only) argument
-  if (!locate_tile<SYMMETRIC>(ka, blockIdx.x, pi, bi, bj)) return;  // padding id of the last eighth: the whole workgroup leaves
+  table_ptr_t ka;
+  if (!locate_tile<SYMMETRIC>(table, blockIdx.x, ka, pi, bi, bj)) return;  // an id past the end of its XCD's list: the whole workgroup leaves
   Problem g;
-  g.A = ka->p[pi].A; g.B = ka->p[pi].B; g.C = ka->p[pi].C; g.C2 = ka->p[pi].C2; g.F = ka->p[pi].F;
-  g.K = ka->p[pi].K; g.lda = ka->p[pi].lda; g.ldb = ka->p[pi].ldb; g.ldc = ka->p[pi].ldc; g.ldc2 = ka->p[pi].ldc2; g.ldf = ka->p[pi].ldf;
-  g.f_rows = ka->p[pi].f_rows; g.f_cols = ka->p[pi].f_cols; g.f_transposed = ka->p[pi].f_transposed; g.scale = ka->p[pi].scale;
-  g.mul_c = ka->p[pi].mul_c; g.diag = ka->p[pi].diag;
+  g.A = ka[pi].A; g.B = ka[pi].B; g.C = ka[pi].C; g.C2 = ka[pi].C2; g.F = ka[pi].F;
+  g.K = ka[pi].K; g.lda = ka[pi].lda; g.ldb = ka[pi].ldb; g.ldc = ka[pi].ldc; g.ldc2 = ka[pi].ldc2; g.ldf = ka[pi].ldf;
+  g.f_rows = ka[pi].f_rows; g.f_cols = ka[pi].f_cols; g.f_transposed = ka[pi].f_transposed; g.scale = ka[pi].scale;
+  g.mul_c = ka[pi].mul_c; g.diag = ka[pi].diag; g.round_out = ka[pi].round_out;
   const int row0 = bi * BM, col0 = bj * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -370,7 +388,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const GroupArgs 
     }
   }
 
-  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj);
+  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, row0, col0, wm, wn, lane, bi, bj);
 }
 
 // The 256 x 256 tile class: four wavefronts of 128 x 128 (one per SIMD, accumulators in the accumulation registers),
@@ -395,7 +413,7 @@ __device__ __forceinline__ bf16x8 lds_read_b128_off(uint32_t addr) {
 }
 
 template <int MODE>
-__global__ __launch_bounds__(256) void ns_gemm4_kernel(const GroupArgs grp) {
+__global__ __launch_bounds__(256) void ns_gemm4_kernel(const void* table) {
   constexpr int BM = 256, BN = 256, BK = 32, STAGES = 4, WGN = 2;
   constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
   constexpr int ROWB = BK * 2;                  // bytes per LDS row
@@ -403,15 +421,15 @@ __global__ __launch_bounds__(256) void ns_gemm4_kernel(const GroupArgs grp) {
   constexpr int LOADS = 8;                      // direct-to-LDS loads (16 rows each) per wavefront and K-tile: 128 rows of one operand
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
+  constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2 || MODE == kModePartial;  // the tile list is the upper triangle
   int pi, bi, bj;
-  const group_ptr_t ka = (group_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
-  if (!locate_tile<SYMMETRIC>(ka, blockIdx.x, pi, bi, bj)) return;
+  table_ptr_t ka;
+  if (!locate_tile<SYMMETRIC>(table, blockIdx.x, ka, pi, bi, bj)) return;
   Problem g;
-  g.A = ka->p[pi].A; g.B = ka->p[pi].B; g.C = ka->p[pi].C; g.C2 = ka->p[pi].C2; g.F = ka->p[pi].F;
-  g.K = ka->p[pi].K; g.lda = ka->p[pi].lda; g.ldb = ka->p[pi].ldb; g.ldc = ka->p[pi].ldc; g.ldc2 = ka->p[pi].ldc2; g.ldf = ka->p[pi].ldf;
-  g.f_rows = ka->p[pi].f_rows; g.f_cols = ka->p[pi].f_cols; g.f_transposed = ka->p[pi].f_transposed; g.scale = ka->p[pi].scale;
-  g.mul_c = ka->p[pi].mul_c; g.diag = ka->p[pi].diag;
+  g.A = ka[pi].A; g.B = ka[pi].B; g.C = ka[pi].C; g.C2 = ka[pi].C2; g.F = ka[pi].F;
+  g.K = ka[pi].K; g.lda = ka[pi].lda; g.ldb = ka[pi].ldb; g.ldc = ka[pi].ldc; g.ldc2 = ka[pi].ldc2; g.ldf = ka[pi].ldf;
+  g.f_rows = ka[pi].f_rows; g.f_cols = ka[pi].f_cols; g.f_transposed = ka[pi].f_transposed; g.scale = ka[pi].scale;
+  g.mul_c = ka[pi].mul_c; g.diag = ka[pi].diag; g.round_out = ka[pi].round_out;
   const int row0 = bi * BM, col0 = bj * BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
@@ -567,7 +585,7 @@ __global__ __launch_bounds__(256) void ns_gemm4_kernel(const GroupArgs grp) {
     if (kt + 3 < KT) tile(kt + 3, ns_ic<3>{}, std::false_type{});
   }
 
-  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, grp.round_out, row0, col0, wm, wn, lane, bi, bj);
+  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, row0, col0, wm, wn, lane, bi, bj);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -585,13 +603,13 @@ struct PrepItem {
   int n_blocks, block_begin;  // sum of squares: this matrix owns workgroups [block_begin, block_begin + n_blocks)
   int tiles_c, tile_begin;    // conversion: 64 x 64 tiles, tiles_c per tile row, first workgroup id
   int legacy;                 // two stochastic rounds (legacy_zeropower_via_newtonschulz5) instead of one
+  int bf16_update;  // the reference's update buffer is bf16: norm and quotient are bf16 values (to nearest), no stochastic round
 };
 constexpr int kMaxPrep = 28;
 struct PrepGroup {
   PrepItem it[kMaxPrep];
   int n_items;
   float eps;
-  int bf16_update;  // the reference's update buffer is bf16: norm and quotient are bf16 values (to nearest), no stochastic round
   Rng rng;
 };
 static_assert(sizeof(PrepGroup) <= 4096, "the group travels as a kernel argument");
@@ -638,7 +656,7 @@ __global__ __launch_bounds__(256) void ns_norm_final_kernel(const PrepGroup grp)
   if (threadIdx.x == 0) {
     float nrm = __builtin_sqrtf((float)(lds[0] + lds[1] + lds[2] + lds[3]));
     float eps = grp.eps;
-    if (grp.bf16_update) {  // a bf16 tensor's norm is a bf16 value; so is the clamp bound, except under the legacy schedule, whose
+    if (ka->it[pi].bf16_update) {  // a bf16 tensor's norm is a bf16 value; so is the clamp bound, except under the legacy schedule, whose
       nrm = bf16_to_f32(f32_to_bf16_rne(nrm));  // division promotes both sides to fp32 first (heavyball/utils.py:1174-1179, :1190)
       if (!ka->it[pi].legacy) eps = bf16_to_f32(f32_to_bf16_rne(eps));
     }
@@ -680,7 +698,7 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
   const int rows = ka->it[pi].rows, cols = ka->it[pi].cols, transpose = ka->it[pi].transpose;
   const int64_t flat_base = ka->it[pi].flat_base;
   // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input), 3: bf16 input under the legacy schedule (one, after the division)
-  const int legacy = grp.bf16_update ? (ka->it[pi].legacy ? 3 : 2) : ka->it[pi].legacy;
+  const int legacy = ka->it[pi].bf16_update ? (ka->it[pi].legacy ? 3 : 2) : ka->it[pi].legacy;
   const Rng rng = grp.rng;
   __shared__ uint16_t tile[64][64 + 8];  // +8: rows 144 B apart, so the column reads below spread over the banks
   const float nrm = ka->it[pi].norm[0];
@@ -744,18 +762,41 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
 static inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 // S = X X^T from its K chunks (added in chunk order) with the epilogue of the one-piece product: S rounded to bf16,
-// Y = c S + b I with one bf16 rounding per operation (heavyball/utils.py:568-570).
-__global__ __launch_bounds__(256) void ns_split_reduce_kernel(const float* __restrict__ part, int chunks, int mp, uint16_t* __restrict__ S,
+// Y = c S + b I with one bf16 rounding per operation (heavyball/utils.py:568-570).  The chunks hold the tiles on and above
+// the diagonal; an element below takes the sum of its mirror image, which has the same terms in the same order.
+__global__ __launch_bounds__(256) void ns_split_reduce_kernel(const float* __restrict__ part, int chunks, int mp, int tile, uint16_t* __restrict__ S,
                                                               uint16_t* __restrict__ Y, float mul_c, float diag) {
+  // one workgroup per 32 x 32 block of a tile on or above the diagonal; a block of a tile above it is also written mirrored,
+  // through LDS, so that both copies leave as runs of 32 elements
+  const int nb = mp / 32;
+  const int br = blockIdx.x / nb, bc = blockIdx.x % nb;
+  const int tr = br * 32 / tile, tc = bc * 32 / tile;
+  if (tr > tc) return;
+  __shared__ uint32_t lds[32][33];
   const int64_t n = (int64_t)mp * mp;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+  const int lc = threadIdx.x & 31, lr0 = (threadIdx.x >> 5) * 4;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int r = br * 32 + lr0 + k, col = bc * 32 + lc;
+    const int64_t i = (int64_t)r * mp + col;
     float v = 0.0f;
     for (int c = 0; c < chunks; ++c) v += part[(size_t)c * n + i];
     const uint32_t h = f32_to_bf16_rne(v);
     uint32_t y = f32_to_bf16_rne(bf16_to_f32(h) * mul_c);
-    if (i / mp == i % mp) y = f32_to_bf16_rne(bf16_to_f32(y) + diag);
+    if (r == col) y = f32_to_bf16_rne(bf16_to_f32(y) + diag);
     S[i] = (uint16_t)h;
     Y[i] = (uint16_t)y;
+    lds[lr0 + k][lc] = h | (y << 16);
+  }
+  if (tr == tc) return;  // wave-uniform: the whole workgroup leaves
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int col = lr0 + k, r = lc;  // element (r, col) of the block goes to (col, r) of the mirrored block
+    const uint32_t w = lds[r][col];
+    const int64_t i = (int64_t)(bc * 32 + col) * mp + br * 32 + r;
+    S[i] = (uint16_t)(w & 0xFFFFu);
+    Y[i] = (uint16_t)(w >> 16);
   }
 }
 
@@ -800,17 +841,19 @@ static NsPlan make_plan(int64_t rows, int64_t cols, int tile) {
   p.off_norm = take(256);
   // A short, very wide X (an embedding matrix under a small hidden size) gives S = X X^T a handful of tiles with a k-loop
   // of hundreds of steps each: a few workgroups work for a long time while the rest of the chip idles.  Such a product is
-  // cut along K into enough chunks for about two workgroups per compute unit; the chunks leave raw fp32 partial products
-  // (all tiles, no mirroring) and ns_split_reduce_kernel adds them up and applies the epilogue of the one-piece product.
+  // cut along K into enough chunks for about two workgroups per compute unit (a multiple of 8 chunks where that many fit:
+  // on the 128-wide tiles a chunk stays on one XCD); the chunks leave raw fp32 partial products of the tiles on and above
+  // the diagonal and ns_split_reduce_kernel adds them up, mirrors them and applies the epilogue of the one-piece product.
   // The choice depends on the shape alone, so a matrix gets the same bits in any batch.
   p.split = 0;
   p.split_chunk = 0;
   p.off_split = o;
   const int64_t T = p.mp / p.tile;
   if (T * (T + 1) / 2 <= 40 && p.np >= 8192) {
-    int64_t sk = 512 / (T * T);  // at most two workgroups per compute unit: one more chunk would start a second, almost empty round
+    int64_t sk = 512 / (T * (T + 1) / 2);  // at most two workgroups per compute unit: one more chunk would start a second, almost empty round
     if (sk > p.np / 2048) sk = p.np / 2048;
     if (sk > 64) sk = 64;
+    if (sk > 8) sk &= ~int64_t(7);
     if (sk >= 2) {
       p.split_chunk = (int)round_up((p.np + sk - 1) / sk, 64);
       p.split = (int)((p.np + p.split_chunk - 1) / p.split_chunk);
@@ -822,56 +865,125 @@ static NsPlan make_plan(int64_t rows, int64_t cols, int tile) {
 }
 
 template <int BM, int BN, int BK, int STAGES, int WGM, int WGN, int MODE>
-static int launch_group(const GroupArgs& a, int n_blocks, hipStream_t s) {
+static int launch_group(const void* table, int n_blocks, hipStream_t s) {
   constexpr int smem = STAGES * (BM + BN) * BK * 2;
   static LdsReservation reserved;
   auto kern = ns_gemm_kernel<BM, BN, BK, STAGES, WGM, WGN, MODE>;
   const void* kp = reinterpret_cast<const void*>(kern);
   if (int rc = reserve_lds(reserved, &kp, 1, smem, "hb_ns5")) return rc;
-  kern<<<n_blocks, WGM * WGN * 64, smem, s>>>(a);
+  kern<<<n_blocks, WGM * WGN * 64, smem, s>>>(table);
   return HB_OK;
 }
 
 template <int MODE>
-static int launch_group4(const GroupArgs& a, int n_blocks, hipStream_t s) {
+static int launch_group4(const void* table, int n_blocks, hipStream_t s) {
   constexpr int smem = 4 * (256 + 256) * 32 * 2;
   static LdsReservation reserved;
   auto kern = ns_gemm4_kernel<MODE>;
   const void* kp = reinterpret_cast<const void*>(kern);
   if (int rc = reserve_lds(reserved, &kp, 1, smem, "hb_ns5")) return rc;
-  kern<<<n_blocks, 256, smem, s>>>(a);
+  kern<<<n_blocks, 256, smem, s>>>(table);
   return HB_OK;
 }
 
-// One product of the iteration for every matrix of one tile class: matrices are listed longest K first (the hardware
-// starts workgroups in id order, so the long tiles start first and the short ones fill in behind them) and launched
-// in groups of at most kMaxGroup.
+// A piece of the tables on its way to device memory: it travels as the argument of a one-workgroup kernel, which is the one
+// way to bring host data to the device from a call that may neither allocate nor copy from pageable memory.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kUploadPieces = 248;
+struct UploadArgs {
+  u32x4 data[kUploadPieces];
+  u32x4* dst;
+  int n;
+};
+static_assert(sizeof(UploadArgs) <= 4096, "the piece travels as a kernel argument");
+
+__global__ __launch_bounds__(256) void ns_upload_kernel(const UploadArgs a) {
+  const auto* ka = (const __attribute__((address_space(4))) UploadArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+  const int t = threadIdx.x;
+  if (t < ka->n) ka->dst[t] = ka->data[t];
+}
+
+// The launches of one Newton-Schulz call, collected first and issued after their tables are on the device: `host` holds
+// every table of the call (each 256-byte aligned), `ops` the launches in order (an op is handed the tables' device address).
+struct Stager {
+  std::vector<char> host;
+  std::vector<std::function<int(const char*)>> ops;
+};
+
+// One product of the iteration for every matrix of one tile class, in one launch.  Fills the tile lists of the eight XCDs as
+// described at locate_tile.
+#ifndef HB_NS_WHOLE_MAX
+#define HB_NS_WHOLE_MAX 256  // a matrix of the 128-wide class with at most this many tiles stays on one XCD
+#endif
 template <int MODE>
-static int gemm_stage(std::vector<Problem> probs, int tile, hipStream_t s, int round_out = 0) {
-  constexpr bool symmetric = MODE == kModeS || MODE == kModeY2;
-  std::stable_sort(probs.begin(), probs.end(), [](const Problem& a, const Problem& b) { return a.K > b.K; });
-  for (size_t first = 0; first < probs.size(); first += kMaxGroup) {
-    GroupArgs a{};
-    a.n_problems = (int)std::min<size_t>(kMaxGroup, probs.size() - first);
-    a.round_out = round_out;
-    int blocks = 0;
-    for (int i = 0; i < a.n_problems; ++i) {
-      Problem& q = a.p[i];
-      q = probs[first + i];
-      q.n_tiles = symmetric ? q.tiles_m * (q.tiles_m + 1) / 2 : q.tiles_m * q.tiles_n;
-      q.tile_begin = blocks;
-      blocks += 8 * ((q.n_tiles + 7) / 8);
+static void gemm_stage(Stager& st, std::vector<Problem> probs, int tile, hipStream_t s) {
+  constexpr bool symmetric = MODE == kModeS || MODE == kModeY2 || MODE == kModePartial;
+  auto tiles_of = [](const Problem& q) { return symmetric ? q.tiles_m * (q.tiles_m + 1) / 2 : q.tiles_m * q.tiles_n; };
+  std::stable_sort(probs.begin(), probs.end(), [&](const Problem& a, const Problem& b) { return (int64_t)a.K * tiles_of(a) > (int64_t)b.K * tiles_of(b); });
+  std::vector<Problem> lists[8];
+  int64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (const Problem& q : probs) {
+    const int n = tiles_of(q);
+    if (tile == 128 && n <= HB_NS_WHOLE_MAX) {
+      const int x = (int)(std::min_element(load, load + 8) - load);
+      Problem e = q;
+      e.t0 = 0;
+      e.n_run = n;
+      lists[x].push_back(e);
+      load[x] += (int64_t)n * q.K;
+      continue;
     }
+    const int per = (n + 7) / 8;
+    for (int x = 0; x < 8 && x * per < n; ++x) {
+      Problem e = q;
+      e.t0 = x * per;
+      e.n_run = std::min(per, n - e.t0);
+      lists[x].push_back(e);
+      load[x] += (int64_t)e.n_run * q.K;
+    }
+  }
+  TableHeader hdr{};
+  int longest = 0, entries = 0;
+  for (int x = 0; x < 8; ++x) {
+    std::stable_sort(lists[x].begin(), lists[x].end(), [](const Problem& a, const Problem& b) { return a.K > b.K; });
+    int pos = 0;
+    for (Problem& e : lists[x]) {
+      e.pos_begin = pos;
+      pos += e.n_run;
+    }
+    longest = std::max(longest, pos);
+    hdr.first[x] = entries;
+    entries += (int)lists[x].size();
+  }
+  hdr.first[8] = entries;
+  const size_t at = (st.host.size() + 255) & ~size_t(255);
+  st.host.resize(at + sizeof(TableHeader) + (size_t)entries * sizeof(Problem));
+  std::memcpy(st.host.data() + at, &hdr, sizeof(TableHeader));
+  size_t o = at + sizeof(TableHeader);
+  for (int x = 0; x < 8; ++x) {
+    if (lists[x].empty()) continue;
+    std::memcpy(st.host.data() + o, lists[x].data(), lists[x].size() * sizeof(Problem));
+    o += lists[x].size() * sizeof(Problem);
+  }
+  const int blocks = 8 * longest;
 #ifndef HB_GEMM_CFG_SMALL
 #define HB_GEMM_CFG_SMALL 128, 128, 64, 2, 2, 4
 #endif
-    const int rc = tile == 256 ? launch_group4<MODE>(a, blocks, s) : launch_group<HB_GEMM_CFG_SMALL, MODE>(a, blocks, s);
-    if (rc) return rc;
-  }
-  return HB_OK;
+  st.ops.push_back([=](const char* dev) {
+    return tile == 256 ? launch_group4<MODE>(dev + at, blocks, s) : launch_group<HB_GEMM_CFG_SMALL, MODE>(dev + at, blocks, s);
+  });
 }
 
-// coeffs_host: 15 floats per matrix when per_matrix, else one table of 15; flags likewise (HB_NS_BF16_UPDATE must agree over the batch)
+// Room for the tables of one call: 15 products, each listing every matrix once, or once per K chunk of a split product
+static size_t table_bytes(const std::vector<NsPlan>& plans) {
+  size_t entries = 0;
+  for (const NsPlan& p : plans) entries += p.split > 1 ? p.split : 1;
+  // 5 iterations x (S, split chunks, Y2, X) in two tile classes; a matrix is listed up to eight times (a run per XCD); each
+  // table has a header and is 256-byte aligned
+  return 20 * (8 * entries * sizeof(Problem) + 2 * (256 + sizeof(TableHeader)));
+}
+
+// coeffs_host: 15 floats per matrix when per_matrix, else one table of 15; flags likewise
 static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                             const float* coeffs_host, const int32_t* flags, bool per_matrix, float eps, const float* post_scale,
                             int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
@@ -882,12 +994,8 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return set_error(HB_EINVAL, "%s: workspace must be 256-byte aligned", who);
   auto flag_of = [&](int i) { return flags[per_matrix ? i : 0]; };
   auto coeff_of = [&](int i, int k) { return coeffs_host[(per_matrix ? (size_t)i * 15 : 0) + k]; };
-  const int bf16_update = (flag_of(0) & HB_NS_BF16_UPDATE) != 0;
-  for (int i = 0; i < n_mats; ++i) {
+  for (int i = 0; i < n_mats; ++i)
     if (flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE)) return set_error(HB_EINVAL, "%s: unknown flag bits", who);
-    if (((flag_of(i) & HB_NS_BF16_UPDATE) != 0) != (bf16_update != 0))
-      return set_error(HB_EINVAL, "%s: HB_NS_BF16_UPDATE must be set for every matrix of a call or for none", who);
-  }
   for (int i = 0; i < n_mats; ++i) {
     if (!g[i] || !out[i]) return set_error(HB_EINVAL, "%s: null matrix pointer at %d", who, i);
     if (rows[i] <= 0 || cols[i] <= 0 || rows[i] > (1 << 20) || cols[i] > (1 << 20)) return set_error(HB_EINVAL, "%s: bad shape at %d", who, i);
@@ -902,8 +1010,12 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
     base[i] = static_cast<char*>(workspace) + total;
     total += plans[i].total;
   }
+  const size_t table_room = table_bytes(plans);
+  char* const dev_tables = static_cast<char*>(workspace) + total;  // every plan's size is a multiple of 256
+  total += table_room;
   if ((int64_t)total > workspace_bytes)
     return set_error(HB_EINVAL, "%s: workspace too small (%lld < %lld)", who, (long long)workspace_bytes, (long long)total);
+  Stager st;
   auto X = [&](int i, int k) { return reinterpret_cast<uint16_t*>(base[i] + plans[i].off_x[k]); };
   auto Xt = [&](int i, int k) { return reinterpret_cast<uint16_t*>(base[i] + plans[i].off_xt[k]); };
   auto S = [&](int i) { return reinterpret_cast<uint16_t*>(base[i] + plans[i].off_s); };
@@ -916,7 +1028,6 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
     PrepGroup pg{};
     pg.n_items = std::min(kMaxPrep, n_mats - first);
     pg.eps = eps;
-    pg.bf16_update = bf16_update;
     pg.rng = rng;
     int blocks = 0, tiles = 0;
     for (int k = 0; k < pg.n_items; ++k) {
@@ -935,6 +1046,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
       q.ldxt = (int)p.mp;
       q.transpose = p.rows > p.cols;
       q.legacy = (flag_of(i) & HB_NS_LEGACY) != 0;
+      q.bf16_update = (flag_of(i) & HB_NS_BF16_UPDATE) != 0;
       const int64_t n = p.rows * p.cols;
       q.n_blocks = (int)std::min<int64_t>(1024, (n + 4095) / 4096);
       q.block_begin = blocks;
@@ -989,17 +1101,21 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
           chunks.push_back(q);
         }
       }
-      if (!whole.empty())
-        if (int rc = gemm_stage<kModeS>(whole, t, s)) return rc;
+      if (!whole.empty()) gemm_stage<kModeS>(st, whole, t, s);
       if (!chunks.empty()) {
-        if (int rc = gemm_stage<kModePartial>(chunks, t, s)) return rc;
+        gemm_stage<kModePartial>(st, chunks, t, s);
         for (size_t k = 0; k < idx.size(); ++k) {
           const int i = idx[k];
           const NsPlan& p = plans[i];
           if (p.split == 0) continue;
-          const int64_t n = p.mp * p.mp;
-          ns_split_reduce_kernel<<<(unsigned)std::min<int64_t>(1024, (n + 255) / 256), 256, 0, s>>>(
-              reinterpret_cast<const float*>(base[i] + p.off_split), p.split, (int)p.mp, S(i), Y(i), cc(i), cb(i));
+          const float* parts = reinterpret_cast<const float*>(base[i] + p.off_split);
+          uint16_t *s_out = S(i), *y_out = Y(i);
+          const float mul_c = cc(i), diag = cb(i);
+          const int split = p.split, mp = (int)p.mp;
+          st.ops.push_back([=](const char*) {
+            ns_split_reduce_kernel<<<(unsigned)((mp / 32) * (mp / 32)), 256, 0, s>>>(parts, split, mp, t, s_out, y_out, mul_c, diag);
+            return (int)HB_OK;
+          });
         }
       }
       // Y2 = Y S + a I  (S symmetric: its rows are the K-contiguous operand; Y2 is a polynomial in S, so only the
@@ -1014,7 +1130,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         q.diag = ca(i);
         probs[k] = q;
       }
-      if (int rc = gemm_stage<kModeY2>(probs, t, s)) return rc;
+      gemm_stage<kModeY2>(st, probs, t, s);
       // X = Y2 X  ==  gemm(Y2, X^T)
       for (size_t k = 0; k < idx.size(); ++k) {
         const int i = idx[k];
@@ -1028,12 +1144,27 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         } else {
           q.F = out[i]; q.f_transposed = p.rows > p.cols; q.ldf = (int)p.cols; q.f_rows = (int)p.rows; q.f_cols = (int)p.cols;
           q.scale = post_scale[i];
+          q.round_out = (flag_of(i) & HB_NS_BF16_UPDATE) != 0;
         }
         probs[k] = q;
       }
-      if (int rc = it < 4 ? gemm_stage<kModeX>(probs, t, s) : gemm_stage<kModeFinal>(probs, t, s, bf16_update)) return rc;
+      if (it < 4) gemm_stage<kModeX>(st, probs, t, s);
+      else gemm_stage<kModeFinal>(st, probs, t, s);
     }
   }
+  // the tables go to the device in pieces of a kernel argument each, then the products run
+  if (st.host.size() > table_room) return set_error(HB_EINVAL, "%s: internal error: tables outgrew their room", who);
+  st.host.resize((st.host.size() + 15) & ~size_t(15));
+  for (size_t at = 0; at < st.host.size(); at += sizeof(UploadArgs::data)) {
+    UploadArgs u;
+    const size_t bytes = std::min(sizeof(UploadArgs::data), st.host.size() - at);
+    std::memcpy(u.data, st.host.data() + at, bytes);
+    u.dst = reinterpret_cast<u32x4*>(dev_tables + at);
+    u.n = (int)(bytes / 16);
+    ns_upload_kernel<<<1, 256, 0, s>>>(u);
+  }
+  for (auto& op : st.ops)
+    if (int rc = op(dev_tables)) return rc;
   return check_launch(who);
 }
 
@@ -1047,8 +1178,12 @@ extern "C" int hb_ns5_batched_workspace_bytes(int32_t n_mats, const int64_t* row
   std::vector<int> tile;
   choose_tiles(n_mats, rows, cols, tile);
   int64_t total = 0;
-  for (int i = 0; i < n_mats; ++i) total += (int64_t)make_plan(rows[i], cols[i], tile[i]).total;
-  *bytes = total;
+  std::vector<NsPlan> plans(n_mats);
+  for (int i = 0; i < n_mats; ++i) {
+    plans[i] = make_plan(rows[i], cols[i], tile[i]);
+    total += (int64_t)plans[i].total;
+  }
+  *bytes = total + (int64_t)table_bytes(plans);
   return HB_OK;
 }
 

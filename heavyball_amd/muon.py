@@ -175,8 +175,10 @@ class Muon(HBOptimizer):
                 if not g.is_contiguous() or g.data_ptr() % 16 or g.device != b.device:
                     g = g.to(b.device).clone(memory_format=torch.contiguous_format)
                 by_dtype.setdefault(g.dtype, []).append((i, g))
-            if (self.gradient_clipping is not None or mars) and len(by_dtype) > 1:
-                raise NotImplementedError("gradient_clipping / mars with gradients of several dtypes in one bucket")
+            if set(by_dtype) - {torch.float32, torch.bfloat16}:
+                # a float16 update buffer is normalised in float16 by the reference's Newton-Schulz (heavyball/utils.py:555): the
+                # result then depends on how the device at hand accumulates a float16 norm, which no fixture pins
+                raise NotImplementedError("Muon: float16 gradients (promote=True lifts them to float32 first)")
             for lst in by_dtype.values():
                 lst.sort(key=lambda t: t[0])
             prepared.append((b, items, by_dtype))
@@ -187,8 +189,6 @@ class Muon(HBOptimizer):
             # MARS heads the chain (heavyball/chainable.py:2698-2699, :642-647): a pass of its own leaves the corrected gradients,
             # rounded to the gradient dtype, in the fp32 role "_clip"; clipping and the momentum go on from there
             for b, lst, gdt in work if mars else ():
-                if gdt not in (torch.float32, torch.bfloat16):
-                    raise NotImplementedError(f"mars with {gdt} gradients on the Muon path")
                 self._mars_prologue(L, group, b, lst, gdt, step, mars_a, mars_oma, mom_fmt, k_o)
             for (b, _, gdt), res in zip(work, (yield from self._clip_gradients_gen(L, group, work, step, gathered=mars))):
                 clipped[(id(b), gdt)] = res
@@ -221,10 +221,8 @@ class Muon(HBOptimizer):
                 # every matrix of the bucket goes through Newton-Schulz in the same grouped launches; under the legacy mode the
                 # square ones take the legacy coefficient table and input rounding (heavyball/utils.py:790-795), the others the default
                 # with bf16 gradients the reference's update buffer is bf16 and Newton-Schulz normalises it in bf16
-                gdts = set(by_dtype)
-                if gdts - {torch.float32, torch.bfloat16} or len(gdts) > 1:
-                    raise NotImplementedError("Muon: gradients of one bucket must all be float32 or all bfloat16")
-                ns_flags = _lib.NS_BF16_UPDATE if gdts == {torch.bfloat16} else 0
+                # (per matrix: a bucket may hold gradients of both dtypes)
+                ns_flags = {i: _lib.NS_BF16_UPDATE if gdt == torch.bfloat16 else 0 for gdt, lst in by_dtype.items() for i, _ in lst}
                 mats = []
                 for i, p, _ in items:
                     if p.dim() < 2:
@@ -241,7 +239,7 @@ class Muon(HBOptimizer):
                     scale = (ctypes.c_float * n)(*[max(1, r / c) ** 0.5 for _, r, c in part])  # heavyball/utils.py:808-809
                     base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
                     arr = (ctypes.c_float * (15 * n))(*[x for lg in legacy for x in coeff_tables[lg]])
-                    flag_a = (ctypes.c_int32 * n)(*[ns_flags | int(lg) for lg in legacy])
+                    flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) for (i, _, _), lg in zip(part, legacy)])
                     nbytes = ctypes.c_int64()
                     _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows_a, cols_a, ctypes.byref(nbytes)))
                     ws = self._ws(b.device, nbytes.value)
@@ -293,8 +291,8 @@ class MuonAdamW(Muon, FirstOrder):
     The un-fused ``scale_by_adam`` writes its result into the update buffer, which has the gradient's dtype; for fp32
     gradients that is the same arithmetic as the fused Adam step, so the vectors run on ``hb_fused_step`` under the
     state names of the un-fused transform.  bf16 gradients on the vector route take the step kernel's update-only mode,
-    which rounds the update to bf16 as that buffer does, and ``hb_update_param`` after it; fp16 gradients raise
-    NotImplementedError (``promote=True`` lifts them to fp32 first).
+    which rounds the update to bf16 as that buffer does, and ``hb_update_param`` after it (fp16 gradients likewise, with
+    casts for roundings); fp16 gradients of matrices raise NotImplementedError (``promote=True`` lifts them to fp32 first).
     State names and initialisation sets follow the reference's index walk with the route in place
     (``nesterov_ema_momentum_4`` with {2, 3, 4}, ``exp_avg_exp_avg_4`` under ``nesterov=False``; ``scale_by_adam_exp_avg_0`` /
     ``_exp_avg_sq_0`` with {0}; ``mars_mars_old_grad_6`` and a 6 in both sets under ``mars``).  ``ecc`` / ``storage_dtype`` apply

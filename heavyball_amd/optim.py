@@ -610,13 +610,11 @@ class HBOptimizer(torch.optim.Optimizer):
 
     def _clip_gradients_gen(self, L, group, buckets, step, gathered=False):
         """``gradient_clipping`` (heavyball/chainable.py:2696-2699): the gradients of the group are gathered into the fp32
-        slab role ``_clip``, clipped there (a clip point, see ``_run_gen``) and, for bf16 gradients, rounded back to bf16 the way
-        ``copy_stochastic_`` does (``hb_sr_bf16``).  ``buckets``: [(bucket, [(index, gradient)], gradient dtype)].  Returns,
+        slab role ``_clip``, clipped there (a clip point, see ``_run_gen``) and, for 16-bit gradients, rounded back the way
+        ``copy_stochastic_`` does (bf16: ``hb_sr_bf16``; fp16: a cast).  ``buckets``: [(bucket, [(index, gradient)], gradient dtype)].  Returns,
         per bucket, the slab role and format the step then reads its gradients from.  Three extra passes over the
         gradients: a capability, not a tuned path."""
         for b, lst, gdt in buckets:
-            if gdt not in (torch.float32, torch.bfloat16):
-                raise NotImplementedError(f"gradient_clipping with {gdt} gradients")
             b.slab.role("_clip", torch.float32)
             if not gathered:  # otherwise an earlier pass (MARS) has left the gradients in the role
                 for i, g in lst:
@@ -633,6 +631,13 @@ class HBOptimizer(torch.optim.Optimizer):
                     _lib.check(L.hb_sr_bf16(role.data_ptr(), narrow.data_ptr(), role.numel(), self._rng_mode(), self.rng_seed,
                                             int(step) & 0xFFFFFFFF, _lib.STREAM_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
                 result.append((narrow, torch.bfloat16, keep))
+            elif gdt == torch.float16:
+                # a float16 buffer takes the clipped values through a plain cast (heavyball/utils.py:2363-2370 rounds stochastically
+                # into bfloat16 only); per tensor, since the bucket may hold tensors with gradients of another dtype
+                b.slab.role("_clip16h", torch.float16)
+                for i, _ in lst:
+                    b.slab.view("_clip16h", i).copy_(b.slab.view("_clip", i))
+                result.append((b.slab.role("_clip16h", torch.float16), torch.float16, keep))
             else:
                 result.append((role, torch.float32, keep))
         return result
@@ -990,8 +995,6 @@ class FirstOrder(HBOptimizer):
                 if lst is None:
                     lst = by_dtype[dt] = []
                 lst.append((i, g))
-            if (self.gradient_clipping is not None or unfused) and len(by_dtype) > 1:
-                raise NotImplementedError("gradient_clipping / update_clipping with gradients of several dtypes in one bucket")
             for gdt, lst in by_dtype.items():
                 lst.sort(key=lambda t: t[0])
                 work.append((b, lst, gdt))
@@ -1097,8 +1100,10 @@ class FirstOrder(HBOptimizer):
             elif gdt == torch.float16 and self.update_clipping is not None:
                 # a float16 update buffer takes the clipped values through a plain cast (heavyball/utils.py:2363-2370 rounds
                 # stochastically into bfloat16 only); the values stay in the fp32 role, every one of them a float16 number
-                wide = b.slab.role("_update", torch.float32)
-                wide.copy_(wide.to(torch.float16))
+                b.slab.role("_update", torch.float32)
+                for i, _ in lst:  # this launch's tensors only: the bucket may hold tensors with gradients of another dtype
+                    wide = b.slab.view("_update", i)
+                    wide.copy_(wide.to(torch.float16))
             offsets, numel = b.slab.meta()
             chunks, n_chunks = b.slab.chunks(tuple(i for i, _ in lst))
             ptrs = [0] * len(b.params)

@@ -271,7 +271,9 @@ int hb_ns5_batched(int32_t n_mats, const float* const* g, float* const* out, con
 /* hb_ns5_batched with a coefficient table and a flag word per matrix (coeffs_host: n_mats x 15 floats, flags: n_mats
  * words, both in HOST memory): under zeroth_power_mode = "legacy_newtonschulz" the dispatcher gives square matrices the
  * legacy variant and the others the default one (heavyball/utils.py:790-795), and one call still covers the whole group.
- * HB_NS_BF16_UPDATE must be set for all matrices or for none.  Bit-identical to separate calls per schedule. */
+ * HB_NS_BF16_UPDATE is per matrix as well (a bucket may hold gradients of both dtypes).  Bit-identical to separate calls per
+ * matrix.  The descriptors of the launches are written into the workspace by the call itself, so the number of matrices is not
+ * bounded by what a kernel argument holds. */
 int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                          const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
                          uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,

@@ -443,6 +443,15 @@ CLIP_COMBOS = [
                                                     weight_decay=0.01, mars_gamma=0.5), torch.float32, 1.0),
     ("laprop_mars_both_clips_caution_bf16grad_ecc", "LaProp", dict(mars=True, gradient_clipping="global_l2norm_clip", update_clipping="l2_clip_",
                                                                    caution=True, ecc="bf16+8", mars_gamma=0.5, lr=0.01), torch.bfloat16, 1.0),
+    # float16 gradients under a gradient clip: the clipped values return to the float16 buffer through a cast
+    ("adamw_gradclip_rms_fp16grad", "AdamW", dict(gradient_clipping="rmsnorm_clip_", weight_decay=0.01), torch.float16, 1.0),
+    ("laprop_mars_gradclip_l2_fp16grad_ecc", "LaProp", dict(mars=True, gradient_clipping="l2_clip_", ecc="bf16+8", mars_gamma=0.5), torch.float16, 1.0),
+    # gradients of several dtypes in one bucket (a tuple: dealt out to the tensors in turn): every clip and rounding is per tensor
+    ("adamw_gradclip_global_l2_mixed_grads", "AdamW", dict(gradient_clipping="global_l2norm_clip", weight_decay=0.01),
+     (torch.float32, torch.bfloat16, torch.float16), 1.0),
+    ("laprop_mars_both_clips_caution_mixed_grads", "LaProp", dict(mars=True, gradient_clipping="rmsnorm_clip_", update_clipping="global_rmsnorm_clip",
+                                                                  caution=True, mars_gamma=0.5, lr=0.01), (torch.bfloat16, torch.float32), 1.0),
+    ("adopt_updclip_l2_mixed_grads_ecc", "ADOPT", dict(update_clipping="l2_clip_", ecc="bf16+8"), (torch.float16, torch.float32, torch.bfloat16), 1e-2),
 ]
 
 
@@ -458,9 +467,11 @@ def test_clipping_combinations_match_oracle(case):
     print("case", name, flush=True)
     cls, kind = CLS[cls_name]
     host, params, opt, orc = H.build_pair(cls, kind, RAGGED, kwargs, DEV, rounding="philox")
+    gdts = [gdt[i % len(gdt)] for i in range(len(RAGGED))] if isinstance(gdt, tuple) else [gdt] * len(RAGGED)
+    gdt = torch.bfloat16 if isinstance(gdt, tuple) else gdt  # mixed: the tolerance of the narrowest
     bf16_update = gdt in (torch.bfloat16, torch.float16) and "update_clipping" in kwargs  # a 16-bit update buffer
     for k in range(1, 5):
-        grads = H.make_grads(RAGGED, k, gdt, gscale)
+        grads = [g.to(t) for g, t in zip(H.make_grads(RAGGED, k, torch.float32, gscale), gdts)]
         for p, g in zip(params, grads):
             p.grad = g.to(DEV)
         opt.step()
@@ -490,15 +501,8 @@ def test_clipping_combinations_match_oracle(case):
                 assert ((g_ - w_).abs() <= 2.0**-6 * (w_.abs() + w_.abs().max())).all(), (name, k, i, key)
 
 
-def test_clipping_combinations_that_are_not_built_raise():
+def test_unknown_clip_name_raises():
     p = [torch.nn.Parameter(torch.zeros(8, device=DEV))]
-    p.append(torch.nn.Parameter(torch.zeros(8, device=DEV)))
-    opt = heavyball_amd.AdamW(p, update_clipping="l2_clip_")
-    p[0].grad_dtype = p[1].grad_dtype = None
-    p[0].grad = torch.ones(8, device=DEV, dtype=torch.bfloat16)  # gradients of two dtypes in one bucket under a clip are not built
-    p[1].grad = torch.ones(8, device=DEV)
-    with pytest.raises(NotImplementedError):
-        opt.step()
     with pytest.raises(ValueError):
         heavyball_amd.AdamW(p, gradient_clipping="no_such_clip")
 

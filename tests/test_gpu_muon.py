@@ -116,8 +116,32 @@ def test_ns5_mixed_schedules_in_one_call_equal_one_call_per_matrix():
         print("case", tuple(G.shape), "legacy" if legacy[k] else "default", flush=True)
         alone = run_ns5(G, legacy=legacy[k], rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=bases[k])
         assert torch.equal(outs[k].cpu().view(torch.int32), alone.view(torch.int32)), f"matrix {k} {tuple(G.shape)}"
-    flags[1] |= 2  # HB_NS_BF16_UPDATE on one matrix only: refused
+    # HB_NS_BF16_UPDATE per matrix too (a bucket whose gradients have both dtypes): matrices 1, 2 and 6 are bf16 values
+    for k in (1, 2, 6):
+        flags[k] |= _lib.NS_BF16_UPDATE
+        gs[k].copy_(gs[k].bfloat16().float())
+    _lib.check(L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None))
+    torch.cuda.synchronize()
+    for k in (1, 2, 6, 0, 7):
+        G = gs[k].cpu().bfloat16() if k in (1, 2, 6) else Gs[k]
+        alone = run_ns5(G, legacy=legacy[k], rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=bases[k])
+        assert torch.equal(outs[k].cpu().view(torch.int32), alone.view(torch.int32)), f"mixed update dtypes: matrix {k} {tuple(G.shape)}"
+    flags[0] |= 4  # an unknown flag bit is refused
     assert L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None) != 0
+
+
+def test_ns5_of_a_bucket_with_more_matrices_than_a_kernel_argument_holds():
+    """Sixty matrices in one call (the descriptors of a launch live in a table in device memory, written by the call itself):
+    bit for bit what a call per matrix gives, for the first, the last and a few in between."""
+    gen = torch.Generator().manual_seed(13)
+    shapes = [(96 + 8 * (k % 7), 64 + 32 * (k % 5)) for k in range(58)] + [(1024, 1100), (200, 8500)]
+    Gs = [torch.randn(s, generator=gen) * 1e-2 for s in shapes]
+    bases = [4096 * 8 * k for k in range(len(shapes))]
+    together = run_ns5_batched(Gs, bases=bases)
+    for k in (0, 1, 27, 28, 29, 56, 57, 58, 59):
+        print("case", k, tuple(Gs[k].shape), flush=True)
+        alone = run_ns5(Gs[k], rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=bases[k])
+        assert torch.equal(together[k].view(torch.int32), alone.view(torch.int32)), f"matrix {k} {tuple(Gs[k].shape)}"
 
 
 def test_ns5_mirrored_symmetric_products():
@@ -259,6 +283,9 @@ MUON_VARIANTS = [
     ("bf16_grads_bf16_momentum", dict(storage_dtype="bfloat16", lr=0.02), torch.bfloat16),
     ("heavyball_ecc16_bf16_grads", dict(ecc="bf16+16", nesterov=False, heavyball_momentum=True, lr=0.02), torch.bfloat16),
     ("plain_ema_caution", dict(nesterov=False, caution=True, weight_decay=0.1, lr=0.02), torch.float32),
+    # gradients of both dtypes in one bucket (dealt out in turn): the update buffer, and with it Newton-Schulz' normalisation, is per tensor
+    ("mixed_grads", dict(lr=0.02, weight_decay=0.01), (torch.bfloat16, torch.float32)),
+    ("mixed_grads_mars_ecc_caution", dict(lr=0.02, mars=True, ecc="bf16+8", caution=True), (torch.float32, torch.bfloat16)),
 ]
 
 
@@ -277,7 +304,8 @@ def test_muon_optimizer_matches_oracle(variant, rounding):
     for p in params:
         p.grad_dtype = None
     for k in range(1, 4):
-        grads = H.make_grads(shapes, k, gdt, 1e-2)
+        gdts = [gdt[i % len(gdt)] for i in range(len(shapes))] if isinstance(gdt, tuple) else [gdt] * len(shapes)
+        grads = [g.to(t) for g, t in zip(H.make_grads(shapes, k, torch.float32, 1e-2), gdts)]
         prev = [p.detach().cpu().clone() for p in params]
         prev_o = [p.clone() for p in orc.params]
         for p, g in zip(params, grads):
