@@ -179,11 +179,29 @@ __device__ __forceinline__ void wait_vmcnt(int n) {  // s_waitcnt vmcnt(n) only 
 
 // The epilogue of both product kernels.  Accumulator register r of tile (i, j) of a wavefront holds row
 // (r/4)*8 + (lane/32)*4 + r%4, column lane%32 of the 32 x 32 block.
-template <int MODE, int TM, int TN, int WTM, int WTN>
+//
+// VIA_LDS (the 128-wide class): the row-major bf16 outputs go through a wavefront-private piece of LDS (`stage`, WTM rows of
+// WTN * 2 + 16 bytes) and leave as 16-byte stores, 4 per wavefront and output instead of 32 two-byte ones.  With k-loops of a
+// few hundred the epilogue is a third of a tile's time, and what it costs is the number of store instructions in the queue that
+// the co-resident workgroup's loads share, not their addresses.  The caller has passed a barrier since the last fragment read.
+template <int MODE, int TM, int TN, int WTM, int WTN, bool VIA_LDS = false>
 __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Problem& g, const int row0, const int col0,
-                                            const int wm, const int wn, const int lane, const int bi, const int bj) {
+                                            const int wm, const int wn, const int lane, const int bi, const int bj, char* stage = nullptr) {
   constexpr bool SYMMETRIC = MODE == kModeS || MODE == kModeY2;
+  constexpr bool BF16_OUT = MODE == kModeS || MODE == kModeY2 || MODE == kModeX;
+  constexpr int PITCH = WTN * 2 + 16;
   const int erow = (lane >> 5) * 4, lcol = lane & 31;
+  // the wavefront's WTM x WTN block from `stage` to row-major `base`: a lane moves 16 bytes, WTN / 8 lanes a row
+  auto flush_rows = [&](uint16_t* base, int ld) {
+    constexpr int PPR = WTN / 8;
+    static_assert(WTM * PPR % 64 == 0, "whole wavefront passes");
+#pragma unroll
+    for (int k = 0; k < WTM * PPR / 64; ++k) {
+      const int p = lane + 64 * k, r = p / PPR, part = p % PPR;
+      const uint4 w = *reinterpret_cast<const uint4*>(stage + r * PITCH + part * 16);
+      *reinterpret_cast<uint4*>(base + (size_t)(row0 + wm * WTM + r) * ld + col0 + wn * WTN + part * 8) = w;
+    }
+  };
   // Transposed copies (X^T, the mirror of a symmetric tile).  A lane holds 4 + 4 + 4 + 4 rows of one column, lane + 32 the
   // rows between them; v_permlane32_swap trades halves so that a lane below 32 ends up with rows 0..15 of its column and
   // its partner with rows 16..31, 32 contiguous bytes of the transposed matrix each (64 per column) instead of 8.
@@ -206,6 +224,10 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
     dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
     dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
   };
+  // VIA_LDS in ModeS: two passes, S and then Y, through the one staging block
+  constexpr int PASSES = VIA_LDS && MODE == kModeS ? 2 : 1;
+#pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) {
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -255,6 +277,11 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
             for (int r = 0; r < 4; ++r)
               if (row + r < g.f_rows && col < g.f_cols) g.F[(size_t)(row + r) * g.ldf + col] = o[r];
           }
+        } else if (VIA_LDS) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            *reinterpret_cast<uint16_t*>(stage + (i * 32 + rb4 * 8 + erow + r) * PITCH + (j * 32 + lcol) * 2) =
+                (uint16_t)(pass == 0 ? prim[rb4 * 4 + r] : sec[rb4 * 4 + r]);
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r) g.C[(size_t)(row + r) * g.ldc + col] = (uint16_t)prim[rb4 * 4 + r];
@@ -264,14 +291,18 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
           }
         }
       }
-      if constexpr (MODE == kModeX) store_transposed(g.C2, g.ldc2, col, row_tile, prim);  // X^T, the B operand of the next iteration
-      // Symmetric modes: a tile above the diagonal is also written transposed to its place below it.  Diagonal tiles
-      // are computed in full, so a matrix that fits one tile gets the plain product.
-      if (SYMMETRIC && bi != bj) {
-        store_transposed(g.C, g.ldc, col, row_tile, prim);
-        if constexpr (MODE == kModeS) store_transposed(g.C2, g.ldc2, col, row_tile, sec);
+      if (pass == 0) {
+        if constexpr (MODE == kModeX) store_transposed(g.C2, g.ldc2, col, row_tile, prim);  // X^T, the B operand of the next iteration
+        // Symmetric modes: a tile above the diagonal is also written transposed to its place below it.  Diagonal tiles
+        // are computed in full, so a matrix that fits one tile gets the plain product.
+        if (SYMMETRIC && bi != bj) {
+          store_transposed(g.C, g.ldc, col, row_tile, prim);
+          if constexpr (MODE == kModeS) store_transposed(g.C2, g.ldc2, col, row_tile, sec);
+        }
       }
     }
+  }
+  if constexpr (VIA_LDS && BF16_OUT) flush_rows(pass == 0 ? g.C : g.C2, pass == 0 ? g.ldc : g.ldc2);
   }
 }
 
@@ -388,7 +419,13 @@ __global__ __launch_bounds__(WGM* WGN * 64) void ns_gemm_kernel(const void* tabl
     }
   }
 
-  ns_epilogue<MODE, TM, TN, WTM, WTN>(acc, g, row0, col0, wm, wn, lane, bi, bj);
+#ifndef HB_NS_EPILOGUE_LDS
+#define HB_NS_EPILOGUE_LDS 1
+#endif
+  constexpr bool kStaged = HB_NS_EPILOGUE_LDS && (MODE == kModeS || MODE == kModeY2 || MODE == kModeX);
+  static_assert(!kStaged || NW * WTM * (WTN * 2 + 16) <= STAGES * STAGE, "the staging blocks reuse the ring");
+  if (kStaged) __syncthreads();  // everyone has read its last fragments: the ring is free
+  ns_epilogue<MODE, TM, TN, WTM, WTN, kStaged>(acc, g, row0, col0, wm, wn, lane, bi, bj, smem + wave * (WTM * (WTN * 2 + 16)));
 }
 
 // The 256 x 256 tile class: four wavefronts of 128 x 128 (one per SIMD, accumulators in the accumulation registers),
