@@ -1011,6 +1011,23 @@ static void gemm_stage(Stager& st, std::vector<Problem> probs, int tile, hipStre
   });
 }
 
+// The tables go to the device in pieces of a kernel argument each, then the launches run in order.
+static int run_staged(Stager& st, char* dev_tables, size_t room, hipStream_t s, const char* who) {
+  if (st.host.size() > room) return set_error(HB_EINVAL, "%s: internal error: tables outgrew their room", who);
+  st.host.resize((st.host.size() + 15) & ~size_t(15));
+  for (size_t at = 0; at < st.host.size(); at += sizeof(UploadArgs::data)) {
+    UploadArgs u;
+    const size_t bytes = std::min(sizeof(UploadArgs::data), st.host.size() - at);
+    std::memcpy(u.data, st.host.data() + at, bytes);
+    u.dst = reinterpret_cast<u32x4*>(dev_tables + at);
+    u.n = (int)(bytes / 16);
+    ns_upload_kernel<<<1, 256, 0, s>>>(u);
+  }
+  for (auto& op : st.ops)
+    if (int rc = op(dev_tables)) return rc;
+  return check_launch(who);
+}
+
 // Room for the tables of one call: 15 products, each listing every matrix once, or once per K chunk of a split product
 static size_t table_bytes(const std::vector<NsPlan>& plans) {
   size_t entries = 0;
@@ -1189,20 +1206,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
       else gemm_stage<kModeFinal>(st, probs, t, s);
     }
   }
-  // the tables go to the device in pieces of a kernel argument each, then the products run
-  if (st.host.size() > table_room) return set_error(HB_EINVAL, "%s: internal error: tables outgrew their room", who);
-  st.host.resize((st.host.size() + 15) & ~size_t(15));
-  for (size_t at = 0; at < st.host.size(); at += sizeof(UploadArgs::data)) {
-    UploadArgs u;
-    const size_t bytes = std::min(sizeof(UploadArgs::data), st.host.size() - at);
-    std::memcpy(u.data, st.host.data() + at, bytes);
-    u.dst = reinterpret_cast<u32x4*>(dev_tables + at);
-    u.n = (int)(bytes / 16);
-    ns_upload_kernel<<<1, 256, 0, s>>>(u);
-  }
-  for (auto& op : st.ops)
-    if (int rc = op(dev_tables)) return rc;
-  return check_launch(who);
+  return run_staged(st, dev_tables, table_room, s, who);
 }
 
 }  // namespace hb
@@ -1222,6 +1226,31 @@ extern "C" int hb_ns5_batched_workspace_bytes(int32_t n_mats, const int64_t* row
   }
   *bytes = total + (int64_t)table_bytes(plans);
   return HB_OK;
+}
+
+extern "C" int hb_ns_product(int32_t tile, int32_t mode, const void* A, const void* B, void* C, void* C2, int64_t M, int64_t N, int64_t K, float mul_c,
+                             float diag, void* workspace, int64_t workspace_bytes, void* stream_) {
+  using namespace hb;
+  if (tile != 128 && tile != 256) return set_error(HB_EINVAL, "hb_ns_product: tile is 128 or 256");
+  if (mode != kModeS && mode != kModeY2 && mode != kModeX) return set_error(HB_EINVAL, "hb_ns_product: mode is 0 (S), 1 (Y2) or 2 (X)");
+  if (!A || !B || !C || !workspace || (mode != kModeY2 && !C2)) return set_error(HB_EINVAL, "hb_ns_product: null pointer");
+  if (M <= 0 || N <= 0 || K <= 0 || M % tile || N % tile || K % 64 || M > (1 << 20) || N > (1 << 20) || K > (1 << 20))
+    return set_error(HB_EINVAL, "hb_ns_product: M and N must be multiples of the tile, K of 64");
+  if (mode != kModeX && M != N) return set_error(HB_EINVAL, "hb_ns_product: the symmetric products are square");
+  if (workspace_bytes < 4096 || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
+    return set_error(HB_EINVAL, "hb_ns_product: the workspace is 4096 bytes, 256-byte aligned");
+  Problem q{};
+  q.A = static_cast<const uint16_t*>(A); q.B = static_cast<const uint16_t*>(B);
+  q.C = static_cast<uint16_t*>(C); q.C2 = static_cast<uint16_t*>(C2);
+  q.K = (int)K; q.lda = (int)K; q.ldb = (int)K; q.ldc = (int)N; q.ldc2 = mode == kModeX ? (int)M : (int)N;
+  q.mul_c = mul_c; q.diag = diag;
+  q.tiles_m = (int)(M / tile); q.tiles_n = (int)(N / tile);
+  hipStream_t s = static_cast<hipStream_t>(stream_);
+  Stager st;
+  if (mode == kModeS) gemm_stage<kModeS>(st, {q}, tile, s);
+  else if (mode == kModeY2) gemm_stage<kModeY2>(st, {q}, tile, s);
+  else gemm_stage<kModeX>(st, {q}, tile, s);
+  return run_staged(st, static_cast<char*>(workspace), 4096, s, "hb_ns_product");
 }
 
 extern "C" int hb_ns5_workspace_bytes(int64_t rows, int64_t cols, int64_t* bytes) {

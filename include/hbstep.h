@@ -279,6 +279,15 @@ int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* ou
                          uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                          void* stream);
 
+/* Test hook: ONE product of the Newton-Schulz iteration on bf16 operands (row-major, K contiguous: A [M, K], B [N, K]) through
+ * the kernel of the given tile class (128 or 256), so that a test can put the same product through both kernels, whose
+ * accumulation order is the same and whose results must agree bit for bit.  mode 0: C = bf16(A B^T), C2 = bf16(bf16(C * mul_c) +
+ * diag on the diagonal) (heavyball/utils.py:568-570; A == B, M == N: upper triangle of tiles computed, mirrored); mode 1:
+ * C = bf16(A B^T) with diag added on the diagonal (:571-572; M == N, upper triangle computed, mirrored); mode 2: C = bf16(A B^T)
+ * [M, N] and C2 = its transpose [N, M] (:573).  M, N multiples of the tile, K of 64.  workspace: 4096 bytes, 256-byte aligned. */
+int hb_ns_product(int32_t tile, int32_t mode, const void* A, const void* B, void* C, void* C2, int64_t M, int64_t N, int64_t K, float mul_c,
+                  float diag, void* workspace, int64_t workspace_bytes, void* stream);
+
 /*
  * SOAP.  hb_gemm_f32: C[M,N] = op(A) op(B) in fp32 on the matrix cores; op(A) = A^T when trans_a (A given as [K,M]),
  * op(B) = B^T when trans_b (B given as [N,K]); row-major, arbitrary sizes and leading dimensions.  `accumulate` is a

@@ -144,6 +144,43 @@ def test_ns5_of_a_bucket_with_more_matrices_than_a_kernel_argument_holds():
         assert torch.equal(together[k].view(torch.int32), alone.view(torch.int32)), f"matrix {k} {tuple(Gs[k].shape)}"
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_both_product_kernels_return_the_same_bits(mode):
+    """The two product kernels (eight wavefronts on 128 x 128 tiles; four hand-scheduled wavefronts on 256 x 256 tiles whose
+    fragment reads go through inline assembly with manual waits) add into an accumulator in the same order, so the same
+    product must come out bit for bit the same from both: a register read ahead of its wait, which the compiler cannot
+    diagnose, would show here.  To be re-run whenever the compiler or a tuning macro of the kernels changes.
+    Mode 1 mirrors the tiles above the diagonal, whose size differs between the kernels: compared where both computed directly."""
+    L = _lib.lib()
+    M, N, K = ((1024, 1024, 2304), (1024, 1024, 1024), (1024, 2304, 1024))[mode]
+    gen = torch.Generator().manual_seed(40 + mode)
+    A = (torch.randn(M, K, generator=gen) * 0.05).bfloat16().to(DEV)
+    B = A if mode == 0 else (torch.randn(N, K, generator=gen) * 0.05).bfloat16().to(DEV)
+    ws = torch.empty(4096, dtype=torch.uint8, device=DEV)
+    out = {}
+    for tile in (128, 256):
+        print("case mode", mode, "tile", tile, flush=True)
+        C = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        C2 = torch.full((N, M) if mode == 2 else (M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        _lib.check(L.hb_ns_product(tile, mode, A.data_ptr(), B.data_ptr(), C.data_ptr(), C2.data_ptr(), M, N, K, 2.5, -3.25, ws.data_ptr(), 4096, None))
+        torch.cuda.synchronize()
+        out[tile] = (C.cpu().view(torch.int16), C2.cpu().view(torch.int16))
+    want = (A.float() @ B.float().T).cpu()
+    got = out[128][0].view(torch.bfloat16).float()
+    direct = (torch.arange(M)[:, None] // 128) <= (torch.arange(N)[None, :] // 128)
+    if mode == 1:
+        want = want + torch.eye(M) * -3.25
+        assert torch.equal(out[128][0][direct], out[256][0][direct])
+        assert ((got - want).abs()[direct] <= 2.0**-7 * want.abs()[direct] + 1e-3).all()
+        return
+    assert torch.equal(out[128][0], out[256][0]) and torch.equal(out[128][1], out[256][1])
+    assert ((got - want).abs() <= 2.0**-7 * want.abs() + 1e-3).all()
+    if mode == 2:
+        assert torch.equal(out[128][1], out[128][0].T)
+    else:
+        assert torch.equal(out[128][0], out[128][0].T)  # S mirrors exactly
+
+
 def test_ns5_mirrored_symmetric_products():
     """Only the upper triangle of tiles of X X^T and of Y S is computed and mirrored; the output has to be what the full
     products give within the Newton-Schulz tolerance on matrices with off-diagonal tiles in both tile classes."""
