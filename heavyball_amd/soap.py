@@ -11,7 +11,9 @@ Householder's up to column signs, which the step is invariant to) and falls back
 numerically rank-deficient; ``eigh`` stays in torch.
 
 With ``split`` a parameter larger than max_precond_dim in some dimension is preconditioned block by block, every block with a
-state of its own under ``state[p][k]`` (heavyball/utils.py:274-286, :1612-1623).
+state of its own under ``state[p][k]`` (heavyball/utils.py:274-286, :1612-1623); what the chain keeps or counts outside the
+preconditioner (MARS' old gradient, the correction of an ECC parameter, caution's count, the per-tensor norms of the clips) is
+per block then as well.
 
 State layout of the reference: ``scale_by_soap_exp_avg_2`` / ``scale_by_soap_exp_avg_sq_2`` with a leading bucket
 dimension of 1, ``scale_by_soap_Q_3`` / ``scale_by_soap_GG_3`` as lists with one ``[1, d, d]`` tensor (or None) per dimension.
@@ -156,14 +158,68 @@ class SOAP(HBOptimizer):
         del defaults["precond_scheduler"]
         self.precond_schedule = 1 / defaults.pop("precondition_frequency")  # heavyball/__init__.py:842-858
         # precond_grad_accum is read by PSGD's guard only (heavyball/chainable.py:304-345): SOAP's chain ignores it, and so does this
-        if split and merge_dims and (mars or caution or param_ecc or ecc or storage_dtype != "float32"):
-            # one state per block (heavyball/utils.py:274-286, :1612-1623): built for the preconditioner's own state in fp32; state
-            # outside it (MARS' old gradient), narrow storage and the per-block count of caution are not
-            raise NotImplementedError("SOAP on the HIP kernels: split together with mars, caution, ecc, param_ecc or non-fp32 storage")
+        self._block_copies = []  # per-block state entries that cannot be views of their slab role: refreshed after every step
         super().__init__(params, defaults, gradient_clipping, update_clipping, palm)
-        per_tensor = ("l2_clip_", "rmsnorm_clip_")
-        if split and merge_dims and (self.gradient_clipping in per_tensor or self.update_clipping in per_tensor):
-            raise NotImplementedError("SOAP on the HIP kernels: split together with clipping by a norm per tensor (per block in the reference)")
+
+    def _adopt_group(self, gi, group):
+        super()._adopt_group(gi, group)
+        if group.get("param_ecc"):  # heavyball/chainable.py:2438-2444: one correction tensor per view of the parameter
+            for b in self._buckets[gi]:
+                for i, p in enumerate(b.params):
+                    self._expose_blocks(group, b, i, p, ("param::ecc",))
+
+    # -- split: state outside the preconditioner, per block ----------------------------------------------------------------
+    # With split the reference runs its whole chain per block (heavyball/utils.py:1612-1623), so MARS' old gradient, the
+    # correction of an ECC parameter, caution's count and the per-tensor norms of the clips are per block.  The kernels keep
+    # working on whole parameters: the old gradient and the correction stay slab roles in the parameter's own layout (both are
+    # elementwise), and ``state[p][k]`` shows block k of them; counts and norms per block are taken with torch on block views.
+    def _blocks_of(self, group, p):
+        """None, or ``[(slices into the merged view, block shape)]`` for a parameter that split cuts up."""
+        if not (group.get("merge_dims", True) and group.get("split") and p.dim() > 0):
+            return None
+        return split_blocks(p.shape, group["max_precond_dim"])
+
+    def _expose_blocks(self, group, b, i, p, keys, value=None):
+        """``state[p][k][key]`` = block k of the slab role ``key`` for a parameter that split cuts up (True), nothing otherwise
+        (False): a view where the block's own shape can be one, else a copy that ``_refresh_block_copies`` keeps current.
+        ``value``: {key: {k: tensor}} to write into the role first (a loaded checkpoint)."""
+        blocks = self._blocks_of(group, p)
+        if blocks is None:
+            return False
+        merged = merged_shape(p.shape, group["max_precond_dim"])
+        self._block_copies = [c for c in self._block_copies if not (c[2] is b and c[3] == i and c[1] in keys)]
+        for k, (where, bshape) in enumerate(blocks):
+            st = self.state[p].setdefault(k, {})
+            for key in keys:
+                if not b.slab.has(key):
+                    continue
+                part = b.slab.view(key, i).reshape(merged)[where]
+                if value is not None and k in value.get(key, {}):
+                    part.copy_(value[key][k].to(part.dtype).reshape(part.shape))
+                try:
+                    st[key] = part.view(bshape or [1])
+                except RuntimeError:  # the block's shape merges dimensions that are strided in the parameter
+                    st[key] = part.reshape(bshape or [1])
+                    self._block_copies.append((st, key, b, i, tuple(merged), where, tuple(bshape or [1])))
+        return True
+
+    def _refresh_block_copies(self):
+        for st, key, b, i, merged, where, bshape in self._block_copies:
+            st[key] = b.slab.view(key, i).reshape(merged)[where].reshape(bshape)
+
+    @staticmethod
+    def _per_block(view, blocks, fn):
+        """``fn(block)`` in place on every block of a tensor's merged view."""
+        for where, _ in blocks:
+            fn(view[where])
+
+    @staticmethod
+    def _clip_block_(kind):
+        """heavyball/utils.py:3226-3262 on one view, in place: the per-tensor clips, which split takes per block."""
+        def clip(x):
+            norm = x.norm() if kind == "l2_clip_" else x.square().mean().sqrt()
+            x.mul_(1.0 / norm.clamp(min=1.0))  # clip_at = 1: clip_at / max(norm, clip_at, eps)
+        return clip
 
     def _run_group(self, gi, group, active):
         active = [(p, g) for p, g in active if p.numel() > 0]  # an empty tensor has nothing to precondition or update
@@ -212,6 +268,11 @@ class SOAP(HBOptimizer):
                 for (i, p, _), g32 in zip(items, raw[key]):
                     st = self._state0(p)
                     if K_OLD not in st:
+                        if self._expose_blocks(group, b, i, p, (K_OLD, K_OLD + "::ecc")):  # split: one old gradient per block
+                            for bst in self.state[p].values():
+                                if isinstance(bst, dict) and K_OLD in bst:
+                                    bst.setdefault("is_initialized", set()).add(5)
+                            continue
                         st[K_OLD] = b.slab.view(K_OLD, i)
                         if mom_corr is not None:
                             st[K_OLD + "::ecc"] = b.slab.view(K_OLD + "::ecc", i)
@@ -227,9 +288,26 @@ class SOAP(HBOptimizer):
         if self.gradient_clipping is not None:
             # heavyball/chainable.py:2696-2699: the clip acts on the update; the gradient itself still initialises the
             # factors (:1235-1238) and is what caution compares against
-            work = [(b, sorted(((i, g32) for (i, _, _), g32 in zip(items, raw[key])), key=lambda t: t[0]), torch.float32)
-                    for key, (b, items) in per_bucket.items()]  # fmt: skip
-            self._clip_gradients(L, group, work, step, gathered=bool(group.get("mars")))
+            # a norm per tensor is a norm per block under split (heavyball/utils.py:1612-1623): those tensors are clipped here,
+            # block by block, and left out of the kernels' clip
+            own = self.gradient_clipping in ("l2_clip_", "rmsnorm_clip_")
+            work = []
+            for key, (b, items) in per_bucket.items():
+                b.slab.role("_clip", torch.float32)
+                lst = []
+                for (i, p, _), g32 in zip(items, raw[key]):
+                    blocks = self._blocks_of(group, p) if own else None
+                    if blocks is None:
+                        lst.append((i, g32))
+                        continue
+                    view = b.slab.view("_clip", i)
+                    if not group.get("mars"):  # otherwise the MARS pass has left the gradient there
+                        view.copy_(g32)
+                    self._per_block(view.reshape(merged_shape(p.shape, max_dim)), blocks, self._clip_block_(self.gradient_clipping))
+                if lst:
+                    work.append((b, sorted(lst, key=lambda t: t[0]), torch.float32))
+            if work:
+                self._clip_gradients(L, group, work, step, gathered=bool(group.get("mars")))
         pending = []  # parameter updates, launched once the (optionally clipped) update of the whole group is there
         for key, (b, items) in per_bucket.items():
             b.slab.role("_update", torch.float32)
@@ -311,15 +389,16 @@ class SOAP(HBOptimizer):
                         continue
                     # split: every block is preconditioned on its own, with its own state (heavyball/utils.py:274-286, :1612-1623);
                     # a block is a strided part of the parameter, so it is gathered, and its update scattered into the slab
-                    done = False
+                    done, start = False, int(b.slab.offsets_np[i])  # the blocks' moments take consecutive runs of the parameter's noise
                     for k, (where, bshape) in enumerate(blocks):
                         bshape = bshape or [1]
                         g0b = G0[where].contiguous().reshape(bshape)
                         gb = g0b if G is G0 else G[where].contiguous().reshape(bshape)
                         ob = torch.empty_like(gb)
-                        if precondition(self.state[p].setdefault(k, {}), g0b, gb, ob, 0):
+                        if precondition(self.state[p].setdefault(k, {}), g0b, gb, ob, start):
                             out[where].copy_(ob.reshape(out[where].shape))
                             done = True
+                        start += gb.numel()
                     if done:
                         updated.append(i)
                 if refresh:
@@ -329,11 +408,49 @@ class SOAP(HBOptimizer):
                             self._narrow(L, job[3], K_M, job[2], mom_fmt, _lib.STREAM_SOAP_ROTATE, step, job[4], stream)
             if updated:
                 pending.append((b, sorted(updated), items, keep))
+        # tensors that split cuts up: their per-tensor update clip and caution's count are per block (torch on block views)
+        cut = {}
+        per_block_clip = self.update_clipping in ("l2_clip_", "rmsnorm_clip_")
+        if group.get("split") and (per_block_clip or group["caution"]):
+            for b, updated, items, keep in pending:
+                for (i, p, _), g32 in zip(items, keep):
+                    blocks = self._blocks_of(group, p) if i in updated else None
+                    if blocks is not None:
+                        cut[(id(b), i)] = (p, g32, blocks)
         if self.update_clipping is not None and pending:  # heavyball/chainable.py:2700-2701
-            clip_keep = self._clip_updates(L, [(b, updated) for b, updated, _, _ in pending])
+            rest = [(b, [i for i in updated if not (per_block_clip and (id(b), i) in cut)]) for b, updated, _, _ in pending]
+            rest = [(b, idx) for b, idx in rest if idx]
+            clip_keep = self._clip_updates(L, rest) if rest else None
+            if per_block_clip:
+                for b, updated, _, _ in pending:
+                    for i in updated:
+                        if (id(b), i) in cut:
+                            p, _, blocks = cut[(id(b), i)]
+                            self._per_block(b.slab.view("_update", i).reshape(merged_shape(p.shape, max_dim)), blocks, self._clip_block_(self.update_clipping))
         else:
             clip_keep = None
+        launches = []
         for b, updated, items, keep in pending:
+            if group["caution"] and any((id(b), i) in cut for i in updated):
+                # heavyball/utils.py:3652-3658 per block, ahead of the parameter update, which then runs without the flag
+                for i in updated:
+                    if (id(b), i) not in cut:
+                        continue
+                    p, g32, blocks = cut[(id(b), i)]
+                    merged = merged_shape(p.shape, max_dim)
+                    uview, gview = b.slab.view("_update", i).reshape(merged), g32.reshape(merged)
+                    for where, _ in blocks:
+                        u, g = uview[where], gview[where]
+                        mask = torch.signbit(g) ^ torch.signbit(u)
+                        u.masked_fill_(mask, 0)
+                        u.mul_(mask.numel() / (mask.numel() - mask.sum()).clamp(min=1))
+                plain = [i for i in updated if (id(b), i) not in cut]
+                if plain:
+                    launches.append((b, plain, items, keep, flags))
+                launches.append((b, [i for i in updated if (id(b), i) in cut], items, keep, flags & ~_lib.FLAG_CAUTION))
+            else:
+                launches.append((b, updated, items, keep, flags))
+        for b, updated, items, keep, flags in launches:
             with torch.cuda.device(b.device):
                 offsets, numel = b.slab.meta()
                 chunks, n_chunks = b.slab.chunks(tuple(updated))
@@ -346,12 +463,13 @@ class SOAP(HBOptimizer):
                 d.grad, d.grad_ptrs = None, table.data_ptr()
                 d.exp_avg = b.slab.ptr("_update")
                 d.offsets, d.numel, d.chunks = offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr()
-                d.caution_count = b.caution_scratch().data_ptr() if group["caution"] else None
+                d.caution_count = b.caution_scratch().data_ptr() if flags & _lib.FLAG_CAUTION else None
                 d.n_chunks, d.n_tensors = n_chunks, len(b.params)
                 d.flags, d.param_fmt, d.grad_fmt = flags, (_lib.ECC_FMT[pecc] if pecc else _PLAIN_FMT[b.param_dtype]), _lib.FMT_F32
                 d.neg_lr, d.one_minus_decay_lr = neg_lr, omdl
                 d.rng_mode, d.step, d.seed = self._rng_mode(), int(step) & 0xFFFFFFFF, self.rng_seed
                 _lib.check(L.hb_update_param(d, current_stream_ptr(b.device)), "hb_update_param")
+        self._refresh_block_copies()
         self._last_launch = (None, [k for *_, k in pending], clip_keep)
 
     def _rehome_state(self):
@@ -360,10 +478,21 @@ class SOAP(HBOptimizer):
         cast is handed over as it is, so a state_dict taken from a live optimizer in the same process would share its moments,
         factors and bases with this one: every state tensor of the preconditioner is copied."""
         super()._rehome_state()
-        for group in self.param_groups:
+        for gi, group in enumerate(self.param_groups):
             for p in group["params"]:
                 if p not in self.state:
                     continue
+                if self._blocks_of(group, p) is not None:
+                    # state outside the preconditioner of a parameter that split cuts up: the loaded blocks go back into their
+                    # slab roles (the parameter's own layout), and state[p][k] shows block k of the role again
+                    keys = [k_ for k_ in (K_OLD, K_OLD + "::ecc", "param::ecc")
+                            if any(isinstance(st, dict) and k_ in st for st in self.state[p].values())]  # fmt: skip
+                    if keys:
+                        b, i = self._find_bucket(gi, p)
+                        for k_ in keys:
+                            b.slab.role(k_, self._role_dtype(group, k_))
+                        value = {k_: {bk: st[k_] for bk, st in self.state[p].items() if isinstance(st, dict) and k_ in st} for k_ in keys}
+                        self._expose_blocks(group, b, i, p, keys, value=value)
                 for st in self.state[p].values():  # block 0, and the further blocks of a split parameter
                     if not isinstance(st, dict):
                         continue

@@ -10,7 +10,8 @@ A ``Rounding`` object answers both for a given (stream, tensor index, shape).  T
                   the magnitude; this is "rounding disabled" and needs no RNG.
   PhiloxRounding  the counter-based stream the kernels use (oracle/philox.py); ``base`` gives each
                   tensor's first flat index in the slab so that element e of tensor t uses counter
-                  base[t] + e.
+                  base[t] + e.  The tensor index may be a pair (t, offsets): the elements of a block of
+                  tensor t, each with its own offset e.
   TorchRounding   torch's global generator in call order: what the reference itself does.
 """
 
@@ -46,8 +47,14 @@ class PhiloxRounding:
 
     def _bits(self, stream, tensor_index, shape):
         n = int(np.prod(shape)) if len(shape) else 1
-        b = 0 if self.base is None else int(self.base[tensor_index])
-        idx = np.arange(b, b + n, dtype=np.uint64)
+        if isinstance(tensor_index, tuple):  # (tensor, offsets of the elements inside it): a block of a tensor that is cut up
+            tensor_index, offsets = tensor_index
+            b = 0 if self.base is None else int(self.base[tensor_index])
+            idx = np.uint64(b) + np.asarray(offsets, dtype=np.uint64)
+            assert idx.size == n
+        else:
+            b = 0 if self.base is None else int(self.base[tensor_index])
+            idx = np.arange(b, b + n, dtype=np.uint64)
         return philox.bits16(self.seed, self.step, stream, idx).reshape(tuple(shape))
 
     def uniform(self, stream, tensor_index, shape):

@@ -11,6 +11,8 @@ is its own bucket here (n = 1), which is also what the reference does for parame
 
 from typing import List, Optional
 
+import numpy as np
+
 import torch
 from torch import Tensor
 
@@ -211,9 +213,7 @@ class SOAPOracle:
         self.mars, self.mars_gamma = mars, mars_gamma
         self.palm, self.beta2_scale, self.merge_dims = palm, beta2_scale, merge_dims
         self.split = split and merge_dims  # heavyball/utils.py:3726-3728: without merge_dims nothing is merged or cut
-        if self.split and (mars or param_ecc is not None or gradient_clipping in ("l2_clip_", "rmsnorm_clip_")
-                           or update_clipping in ("l2_clip_", "rmsnorm_clip_")):  # fmt: skip
-            raise NotImplementedError("split with state or norms per block outside the preconditioner")
+        self.max_precond_dim = max_precond_dim
         self.block_state = [dict() for _ in params]
         self._state_init = [dict() for _ in params]
         if param_ecc is not None:  # heavyball/chainable.py:2421-2444: the live parameter is narrowed at construction
@@ -224,7 +224,9 @@ class SOAPOracle:
                 if p.dtype != pd:
                     e.compute_correction(p.float(), self.rounding.at_step(0).uniform(philox.STREAM_INIT_PARAM, i, p.shape))
                 narrowed.append(e)
-                self._state_init[i]["param::ecc"] = e.corr
+                # heavyball/chainable.py:2438-2444: one correction tensor per view of the parameter, i.e. per block under split
+                for k, blk in enumerate(self._views(e)):
+                    (self._state_init[i] if k == 0 else self.block_state[i].setdefault(k, {}))["param::ecc"] = blk.corr
             params = narrowed
         self.params = params
         self.gradient_clipping, self.update_clipping = gradient_clipping, update_clipping
@@ -253,6 +255,37 @@ class SOAPOracle:
     K_OLD = "mars_mars_old_grad_5"  # pinned by a trajectory written from the reference
     K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
 
+    def _views(self, t):
+        """The views the chain runs on (heavyball/utils.py:1612-1623): the blocks of a split tensor or ECC pair, cut alike; the
+        tensor itself otherwise."""
+        from .ecc import EccTensor
+
+        if not self.split:
+            return [t]
+        if isinstance(t, EccTensor):
+            return [EccTensor(a, b) for a, b in zip(self._views(t.primary), self._views(t.corr))]
+        r = dim_merger(t, self.max_precond_dim, True)
+        return r if isinstance(r, list) else [t]
+
+    def _block_state(self, i, k):
+        return self.state[i] if k == 0 else self.block_state[i].setdefault(k, {})
+
+    def _noise_index(self, i, shape, private=False):
+        """What the rounding is handed as the tensor index of the blocks of parameter i.  Without split: i.  With split, per block,
+        (i, offsets): state that lives in the parameter's own layout (the parameter, its correction, MARS' old gradient) takes the
+        noise of the elements' places in the parameter; the moments of the preconditioner, one tensor per block, take consecutive
+        runs (``private``)."""
+        if not self.split:
+            return [i]
+        idx = self._views(torch.arange(int(np.prod(shape)) if len(shape) else 1).reshape(shape))
+        if not private:
+            return [(i, b.reshape(-1).numpy().astype(np.uint64)) for b in idx]
+        out, start = [], 0
+        for b in idx:
+            out.append((i, np.arange(start, start + b.numel(), dtype=np.uint64)))
+            start += b.numel()
+        return out
+
     def _view_shape(self, shape):
         """heavyball/utils.py:3726-3742: without merge_dims the tensors are taken as they are."""
         return merged_shape(shape, self.max_precond_dim) if self.merge_dims else list(shape)
@@ -273,28 +306,33 @@ class SOAPOracle:
             from . import first_order as fo
 
             keys = list(updates)
-            # zero_guard with the group's storage, like the moments (heavyball/chainable.py:277-301), in the parameter's own shape
-            old = [self._moment(self.state[k], self.K_OLD, grads[k]) for k in keys]
-            fo.mars_correction([updates[k] for k in keys], old, self.mars_gamma, self.betas[0], self.rounding.at_step(int(step)), keys)
+            # zero_guard with the group's storage, like the moments (heavyball/chainable.py:277-301), in the shape of the view the
+            # chain runs on: the parameter's own, or a block's under split (the blocks are views: the correction lands in updates[k])
+            ub, ob, tb = [], [], []
+            for k in keys:
+                for bk, (u, t) in enumerate(zip(self._views(updates[k]), self._noise_index(k, updates[k].shape))):
+                    ub.append(u)
+                    ob.append(self._moment(self._block_state(k, bk), self.K_OLD, u))
+                    tb.append(t)
+            fo.mars_correction(ub, ob, self.mars_gamma, self.betas[0], self.rounding.at_step(int(step)), tb)
             grads = [updates[i].clone() if i in updates else None for i in range(len(grads))]
         if self.gradient_clipping is not None and updates:  # heavyball/chainable.py:2696-2699: on the update, ahead of the transform
             from . import first_order as fo
 
             fn = {"l2_clip_": fo.l2_clip, "rmsnorm_clip_": fo.rmsnorm_clip, "global_l2norm_clip": fo.global_l2norm_clip,
                   "global_rmsnorm_clip": fo.global_rmsnorm_clip}[self.gradient_clipping]  # fmt: skip
-            keys = list(updates)
-            for k, c in zip(keys, fn([updates[k] for k in keys])):
-                updates[k] = c.to(updates[k].dtype)
+            views = [u for k in updates for u in self._views(updates[k])]  # under split the norms are per block
+            for u, c in zip(views, fn(views)):
+                u.copy_(c.to(u.dtype))
         for i, (p, g) in enumerate(zip(self.params, grads)):
             if g is None:
                 continue
-            if self.split:  # blocks of the parameter, of the gradient and of the update, cut alike
-                pv, gv, uv = (dim_merger(t, self.max_precond_dim, True) for t in (p, g, updates[i]))
-                blocks = list(zip(pv, gv, uv)) if isinstance(pv, list) else [(p, g, updates[i])]
-            else:
-                blocks = [(p, g, updates[i])]
+            # blocks of the parameter, of the gradient and of the update, cut alike
+            blocks = list(zip(self._views(p), self._views(g), self._views(updates[i])))
+            private = self._noise_index(i, g.shape, private=True)
+            shared = self._noise_index(i, g.shape)
             for k, (p, g, upd) in enumerate(blocks):
-                st = self.state[i] if k == 0 else self.block_state[i].setdefault(k, {})
+                st = self._block_state(i, k)
                 u = upd.reshape(self._view_shape(g.shape)).unsqueeze(0)  # merged view + the bucket dimension
                 if self.K_M not in st:  # first step: ZeroGuard + GeneralGuard init, no update (heavyball/chainable.py:372-377)
                     self._moment(st, self.K_M, u)
@@ -307,17 +345,17 @@ class SOAPOracle:
                 gp = project(u, Q, False)
                 rounding = self.rounding.at_step(int(step))
                 m_st, v_st = self._moment(st, self.K_M, u), self._moment(st, self.K_V, u)
-                precond = adam_(m_st, v_st, gp, self.betas[0], self.betas[1], step - 1, self.eps, rounding, i)
+                precond = adam_(m_st, v_st, gp, self.betas[0], self.betas[1], step - 1, self.eps, rounding, private[k])
                 precond = project(precond, Q, True)
                 beta = beta_debias(self.shampoo_beta, step)  # heavyball/chainable.py:1244
                 update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta)
                 if is_precond:
-                    gap = refresh_basis(GG, Q, m_st, rounding, i)
+                    gap = refresh_basis(GG, Q, m_st, rounding, private[k])
                     self.sort_key_gap[(i, k)] = min(self.sort_key_gap.get((i, k), 1.0), gap)
                 todo_p.append(p)
                 todo_u.append(precond.squeeze(0).reshape(p.shape))
                 todo_g.append(g)
-                todo_i.append(i)
+                todo_i.append(shared[k])
         if todo_p and self.update_clipping is not None:  # heavyball/chainable.py:2700-2701
             from . import first_order as fo
 

@@ -374,6 +374,23 @@ def make_soap_mars_combinations():
              shapes, torch.float32, 6, grad_scale=3.0)  # fmt: skip
 
 
+def make_soap_split_combinations():
+    """SOAP with split=True together with the switches that keep state or take norms outside the preconditioner: with split the
+    whole chain runs per block (heavyball/utils.py:1612-1623), so MARS' old gradient, caution's count, the per-tensor norms of
+    the clips, narrow moments and the ECC pair of the parameter are all per block.  (20, 12) -> six blocks, (16,) -> two vectors,
+    (6, 30) -> four blocks."""
+    shapes = [(20, 12), (16,), (6, 30)]
+    base = dict(split=True, max_precond_dim=8, precondition_frequency=3)
+    run_traj("soap_split_caution", heavyball.SOAP, dict(base, caution=True, weight_decay=0.1), shapes, torch.float32, 6)
+    run_traj("soap_split_mars", heavyball.SOAP, dict(base, mars=True, mars_gamma=0.1), shapes, torch.float32, 6)
+    run_traj("soap_split_ecc", heavyball.SOAP, dict(base, ecc="bf16+8"), shapes, torch.float32, 6)
+    run_traj("soap_split_bf16_storage", heavyball.SOAP, dict(base, storage_dtype="bfloat16"), shapes, torch.float32, 6)
+    run_traj("soap_split_param_ecc", heavyball.SOAP, dict(base, param_ecc="bf16+8"), shapes, torch.float32, 6)
+    run_traj("soap_split_clip_l2", heavyball.SOAP, dict(base, gradient_clipping="l2_clip_"), shapes, torch.float32, 6, grad_scale=1.0)
+    run_traj("soap_split_updclip_rms_caution", heavyball.SOAP, dict(base, update_clipping="rmsnorm_clip_", caution=True, lr=0.05), shapes,
+             torch.float32, 6)  # fmt: skip
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -531,7 +548,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -556,6 +573,8 @@ if __name__ == "__main__":
         make_muon_narrow_clips()
     if "soapmars" in which:
         make_soap_mars_combinations()
+    if "soapsplit" in which:
+        make_soap_split_combinations()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:

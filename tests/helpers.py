@@ -165,3 +165,21 @@ def run_steps(opt, orc, params, shapes, steps, grad_dtype, grad_scale, device, n
         assert all(p.grad is None for p in params)
         if check_each or k == steps:
             compare(opt, orc, params, f"{tag} step {k}")
+
+
+def whole_from_blocks(d, prefix, key, shape, kwargs):
+    """A per-view state entry of a fixture (``prefix + key`` for block 0, ``prefix + "block<k>/" + key`` for the others) put
+    together in the parameter's own layout; the entry itself when the parameter is not cut."""
+    from oracle.soap import dim_merger
+
+    first = d[prefix + key]
+    if not (kwargs.get("split") and kwargs.get("merge_dims", True)) or tuple(first.shape) == tuple(shape):
+        return first
+    n = 1
+    for s_ in shape:
+        n *= s_
+    places = dim_merger(torch.arange(n).reshape(shape), kwargs.get("max_precond_dim", 2048), True)
+    out = torch.empty(n, dtype=first.dtype)
+    for k, idx in enumerate(places):
+        out[idx.reshape(-1)] = d[prefix + (f"block{k}/" if k else "") + key].reshape(-1)
+    return out.reshape(shape)

@@ -62,6 +62,9 @@ def test_soap_is_adam_in_the_eigenbasis():
     assert torch.allclose(before - orc.params[0], upd, atol=1e-5)
 
 
+from tests.helpers import whole_from_blocks  # noqa: E402
+
+
 @pytest.mark.parametrize("path", TRAJ, ids=[os.path.basename(p)[5:-3] for p in TRAJ])
 def test_soap_trajectory_matches_reference(path):
     d = torch.load(path, weights_only=True)
@@ -73,7 +76,7 @@ def test_soap_trajectory_matches_reference(path):
         for i in range(n):
             want, got = d[f"step{k}/p{i}"], orc.params[i]
             if isinstance(got, EccTensor):  # param_ecc: compare the decoded value, the pair's resolution is 2^-8 of a bf16 ulp
-                want, got = EccTensor(want, d[f"step{k}/state{i}/param::ecc"]).decode(), got.decode()
+                want, got = EccTensor(want, whole_from_blocks(d, f"step{k}/state{i}/", "param::ecc", want.shape, kwargs)).decode(), got.decode()
             assert torch.allclose(got, want, rtol=1e-4, atol=1e-6), (k, i, (got - want).abs().max())
             for key in (orc.K_M, orc.K_V):
                 have, ref = orc.state[i][key], d[f"step{k}/state{i}/{key}"]
@@ -93,14 +96,29 @@ def test_soap_trajectory_matches_reference(path):
             for bk in blocks:
                 st = orc.block_state[i][bk]
                 for key in (orc.K_M, orc.K_V):
-                    ref = d[f"step{k}/state{i}/block{bk}/{key}"]
-                    assert tuple(st[key].shape) == tuple(ref.shape)
-                    assert torch.allclose(st[key], ref, rtol=1e-3, atol=1e-6), (k, i, bk, key)
+                    have, ref = st[key], d[f"step{k}/state{i}/block{bk}/{key}"]
+                    assert tuple(have.shape) == tuple(ref.shape) and have.dtype == ref.dtype
+                    assert (key + "::ecc" in st) == (f"step{k}/state{i}/block{bk}/{key}::ecc" in d)
+                    if key + "::ecc" in st:
+                        have, ref = EccTensor(have, st[key + "::ecc"]).decode(), EccTensor(ref, d[f"step{k}/state{i}/block{bk}/{key}::ecc"]).decode()
+                    tol = 1e-2 if have.dtype == torch.bfloat16 else 1e-3
+                    assert torch.allclose(have.float(), ref.float(), rtol=tol, atol=1e-6), (k, i, bk, key)
                 for li, gg in enumerate(st[orc.K_GG]):
                     gk = f"step{k}/state{i}/block{bk}/{orc.K_GG}/{li}"
                     assert (gg is None) == (gk not in d)
                     if gg is not None:
                         assert torch.allclose(gg, d[gk], rtol=1e-4, atol=1e-8)
+            # state outside the preconditioner, per view of the parameter: MARS' old gradient (a copy of the raw gradient) and the
+            # correction of an ECC parameter (compared through the decoded pair: its resolution is 2^-8 of a bf16 ulp)
+            for bk in [0, *sorted(blocks)]:
+                st = orc.state[i] if bk == 0 else orc.block_state[i][bk]
+                pre = f"step{k}/state{i}/" + (f"block{bk}/" if bk else "")
+                assert (pre + orc.K_OLD in d) == (orc.K_OLD in st), (k, i, bk)
+                if orc.K_OLD in st:
+                    assert tuple(st[orc.K_OLD].shape) == tuple(d[pre + orc.K_OLD].shape) and torch.equal(st[orc.K_OLD], d[pre + orc.K_OLD]), (k, i, bk)
+                assert (pre + "param::ecc" in d) == ("param::ecc" in st), (k, i, bk)
+                if "param::ecc" in st:
+                    assert tuple(st["param::ecc"].shape) == tuple(d[pre + "param::ecc"].shape) and st["param::ecc"].dtype == d[pre + "param::ecc"].dtype
     if "c5" in path:
         assert [s + 1 for s, f in enumerate(orc.fired) if f] == [11]
 
