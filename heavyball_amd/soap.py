@@ -255,8 +255,10 @@ class SOAP(HBOptimizer):
             if b.param_dtype != torch.float32 and not group.get("param_ecc"):
                 raise NotImplementedError("SOAP on the HIP kernels takes fp32 parameters (or param_ecc)")
             if any(g.dtype != torch.float32 for _, _, g in items) and not self.promote:
-                raise NotImplementedError("SOAP on the HIP kernels takes fp32 gradients (the reference rounds every intermediate of a "
-                                          "16-bit update to that dtype); pass promote=True to lift them to fp32 first")  # fmt: skip
+                # the preconditioner itself promotes (heavyball/chainable.py:1261), but the factors and the bases are created in the
+                # gradient's dtype (heavyball/utils.py:1381, :996): bf16 factors, stochastically rounded at every update
+                raise NotImplementedError("SOAP on the HIP kernels takes fp32 gradients (with 16-bit gradients the reference keeps the factors "
+                                          "and the eigenbases in that dtype); pass promote=True to lift them to fp32 first")  # fmt: skip
             raw[key] = [g.to(b.device, torch.float32).contiguous() for _, _, g in items]
             if group.get("mars"):
                 # heavyball/chainable.py:642-647 heads the chain and writes the corrected gradient over the gradient itself: a
