@@ -248,18 +248,26 @@ class SOAP(HBOptimizer):
             b, i = self._find_bucket(gi, p)
             per_bucket.setdefault(id(b), [b, []])[1].append((i, p, g))
         raw: Dict[int, List] = {}
+        gdts: Dict[int, List] = {}  # the dtype of each tensor's update buffer: its gradient's (fp32 under promote)
+        keep_given = []
         for key, (b, items) in per_bucket.items():
             if b.device.type != "cuda":
                 raise _lib.HbError("the optimizer step runs on the GPU only: parameters must live on a CUDA/HIP device")
             self._check_home(b, items)
-            if b.param_dtype != torch.float32 and not group.get("param_ecc"):
-                raise NotImplementedError("SOAP on the HIP kernels takes fp32 parameters (or param_ecc)")
-            if any(g.dtype != torch.float32 for _, _, g in items) and not self.promote:
-                # the preconditioner itself promotes (heavyball/chainable.py:1261), but the factors and the bases are created in the
-                # gradient's dtype (heavyball/utils.py:1381, :996): bf16 factors, stochastically rounded at every update
-                raise NotImplementedError("SOAP on the HIP kernels takes fp32 gradients (with 16-bit gradients the reference keeps the factors "
-                                          "and the eigenbases in that dtype); pass promote=True to lift them to fp32 first")  # fmt: skip
-            raw[key] = [g.to(b.device, torch.float32).contiguous() for _, _, g in items]
+            # 16-bit gradients (without promote): the preconditioner itself promotes what it is handed (heavyball/chainable.py:1261,
+            # :1248), so the gradient's values go through it as fp32; what stays 16-bit is the update buffer ahead of it (MARS and a
+            # gradient clip round into it) and the factors and bases, which are created in the gradient's dtype (gdts, see precondition)
+            given = []
+            for _, _, g in items:
+                if g.is_sparse:
+                    raise NotImplementedError("sparse gradients")
+                if g.dtype not in _PLAIN_FMT or (self.promote and g.dtype != torch.float32):
+                    g = g.float()
+                if g.device != b.device or not g.is_contiguous() or g.data_ptr() % 16:
+                    g = g.to(b.device).clone(memory_format=torch.contiguous_format)
+                given.append(g)
+            gdts[key] = [g.dtype for g in given]
+            raw[key] = [g if g.dtype == torch.float32 else g.float() for g in given]
             if group.get("mars"):
                 # heavyball/chainable.py:642-647 heads the chain and writes the corrected gradient over the gradient itself: a
                 # pass of its own leaves it in the fp32 role "_clip", which then stands for the gradient everywhere below
@@ -279,9 +287,10 @@ class SOAP(HBOptimizer):
                         if mom_corr is not None:
                             st[K_OLD + "::ecc"] = b.slab.view(K_OLD + "::ecc", i)
                         st.setdefault("is_initialized", set()).add(5)
-                raw[key] = [g if g.data_ptr() % 16 == 0 else g.clone() for g in raw[key]]
-                lst = sorted(((i, g32) for (i, _, _), g32 in zip(items, raw[key])), key=lambda t: t[0])
-                self._mars_prologue(L, group, b, lst, torch.float32, step, *mars_weights(group), mom_fmt, K_OLD)
+                for gdt in sorted(set(gdts[key]), key=str):  # the corrected gradient is rounded into the gradient's dtype
+                    lst = sorted(((i, g) for (i, _, _), g in zip(items, given) if g.dtype == gdt), key=lambda t: t[0])
+                    self._mars_prologue(L, group, b, lst, gdt, step, *mars_weights(group), mom_fmt, K_OLD)
+                keep_given.append(given)
                 raw[key] = [b.slab.view("_clip", i) for i, _, _ in items]
                 if self.gradient_clipping is not None:
                     # the clip below rewrites the role in place; what stands for the gradient (the first factors of a tensor's
@@ -293,23 +302,38 @@ class SOAP(HBOptimizer):
             # a norm per tensor is a norm per block under split (heavyball/utils.py:1612-1623): those tensors are clipped here,
             # block by block, and left out of the kernels' clip
             own = self.gradient_clipping in ("l2_clip_", "rmsnorm_clip_")
-            work = []
+            work, own_narrow = [], []
             for key, (b, items) in per_bucket.items():
                 b.slab.role("_clip", torch.float32)
-                lst = []
-                for (i, p, _), g32 in zip(items, raw[key]):
+                lists: Dict[torch.dtype, List] = {}
+                for (i, p, _), g32, gdt in zip(items, raw[key], gdts[key]):
                     blocks = self._blocks_of(group, p) if own else None
                     if blocks is None:
-                        lst.append((i, g32))
+                        lists.setdefault(gdt, []).append((i, g32))
                         continue
                     view = b.slab.view("_clip", i)
                     if not group.get("mars"):  # otherwise the MARS pass has left the gradient there
                         view.copy_(g32)
                     self._per_block(view.reshape(merged_shape(p.shape, max_dim)), blocks, self._clip_block_(self.gradient_clipping))
-                if lst:
-                    work.append((b, sorted(lst, key=lambda t: t[0]), torch.float32))
+                    if gdt != torch.float32:
+                        own_narrow.append((b, i, gdt))
+                for gdt, lst in lists.items():
+                    work.append((b, sorted(lst, key=lambda t: t[0]), gdt))
+            clipped_role = {}
             if work:
-                self._clip_gradients(L, group, work, step, gathered=bool(group.get("mars")))
+                for (b, _, gdt), res in zip(work, self._clip_gradients(L, group, work, step, gathered=bool(group.get("mars")))):
+                    clipped_role[(id(b), gdt)] = res[0]
+            for b, i, gdt in own_narrow:  # the clipped values go back into the 16-bit update buffer (heavyball/utils.py:3231)
+                view = b.slab.view("_clip", i)
+                if gdt == torch.bfloat16:
+                    narrow = torch.empty_like(view, dtype=torch.bfloat16)
+                    with torch.cuda.device(b.device):
+                        _lib.check(L.hb_sr_bf16(view.data_ptr(), narrow.data_ptr(), view.numel(), self._rng_mode(), self.rng_seed,
+                                                int(step) & 0xFFFFFFFF, _lib.STREAM_CLIP, int(b.slab.offsets_np[i]), current_stream_ptr(b.device)),
+                                   "hb_sr_bf16")  # fmt: skip
+                    view.copy_(narrow)
+                else:
+                    view.copy_(view.to(gdt))
         pending = []  # parameter updates, launched once the (optionally clipped) update of the whole group is there
         for key, (b, items) in per_bucket.items():
             b.slab.role("_update", torch.float32)
@@ -317,9 +341,10 @@ class SOAP(HBOptimizer):
             stream = current_stream_ptr(b.device)
             updated, keep, refresh = [], [], []
             with torch.cuda.device(b.device):
-                def precondition(st, G0, G, out, base):
+                def precondition(st, G0, G, out, base, fdt):
                     """One tensor or block: G0 the gradient, G the update that goes through the preconditioner, both in the merged
-                    view; the preconditioned update lands in ``out``.  False on the first step, which only initialises."""
+                    view (fp32 values); the preconditioned update lands in ``out``.  False on the first step, which only initialises.
+                    ``fdt``: the gradient's dtype, which the factors and bases created here take (heavyball/utils.py:1381, :996)."""
                     if K_M not in st:  # first step: initialise, no update (heavyball/chainable.py:372-377, utils.py:1362-1388)
                         for km in (K_M, K_V):  # zero_guard with the group's storage (heavyball/chainable.py:277-301)
                             st[km] = torch.zeros((1, *G.shape), dtype=mom_prim, device=b.device)
@@ -332,6 +357,10 @@ class SOAP(HBOptimizer):
                         else:
                             GG.append(None)
                         self._update_ggt(gemm, G0, GG, 1.0, 0.0)  # beta = 0: a = 1
+                        if fdt != torch.float32:
+                            # 16-bit factors: the first one is the rounded product itself (the reference's contraction of a 16-bit
+                            # gradient returns that dtype, utils.py:1387); the basis below comes from the stored values and is cast (:1003)
+                            GG = [None if m is None else m.to(fdt) for m in GG]
                         Q = []
                         for m in GG:
                             if m is None:
@@ -344,11 +373,11 @@ class SOAP(HBOptimizer):
                             # 0.7 s instead of 0.4 s for an 8192-wide factor, once.
                             eye = torch.eye(m.shape[-1], dtype=torch.float64, device=m.device)
                             _, vec = torch.linalg.eigh(m.double() + 1e-30 * eye)
-                            Q.append(torch.flip(vec, [-1]).to(torch.float32).contiguous())
+                            Q.append(torch.flip(vec, [-1]).to(fdt).contiguous())
                         st[K_GG], st[K_Q] = GG, Q
                         st.setdefault("is_initialized", set()).update({0, 2, 3})
                         return False
-                    Q, GG = st[K_Q], st[K_GG]
+                    GG, Q = self._factors32(st)
                     gp = self._project(gemm, G, Q, back=False)
                     a1, oma1 = debiased_weights(beta1, adam_step)
                     a2, oma2 = debiased_weights(beta2, adam_step)
@@ -369,24 +398,31 @@ class SOAP(HBOptimizer):
                     a = 1 - sb
                     a = a.to(torch.float32) if isinstance(a, torch.Tensor) else f32(a)
                     self._update_ggt(gemm, G, GG, float(a), float(1 - a))
+                    self._store_factors(L, st, K_GG, GG, _lib.STREAM_SOAP_GG, step, base, stream)
                     if is_precond:
                         if mom_fmt == _lib.FMT_F32:
-                            refresh.append((GG, Q, st[K_M]))
+                            refresh.append((GG, Q, st[K_M], st, base))
                         else:  # the rotation reads exp_avg as stored (heavyball/utils.py:883) and writes it back through the codec
                             refresh.append((GG, Q, self._widen(L, st, K_M, mom_fmt, stream), st, base))
                     return True
 
-                for (i, p, g), g32 in zip(items, raw[key]):
+                for (i, p, g), g32, gdt in zip(items, raw[key], gdts[key]):
                     keep.append(g32)
                     # heavyball/utils.py:3726-3742: without merge_dims the parameter is taken as it is
                     merging = group.get("merge_dims", True)
                     shape = (merged_shape(p.shape, max_dim) if merging else list(p.shape)) if p.dim() > 0 else []
                     G0 = g32.reshape(shape) if shape else g32.reshape(1)  # the gradient
-                    G = b.slab.view("_clip", i).reshape(G0.shape) if self.gradient_clipping is not None else G0  # the update
+                    G = G0  # the update
+                    if self.gradient_clipping is not None:
+                        role = clipped_role.get((id(b), gdt))  # a 16-bit role where the kernels' clip rounded into one
+                        if role is not None and role.dtype != torch.float32 and not (own and self._blocks_of(group, p) is not None):
+                            G = b.slab.view("_clip16" if role.dtype == torch.bfloat16 else "_clip16h", i).float().reshape(G0.shape)
+                        else:
+                            G = b.slab.view("_clip", i).reshape(G0.shape)
                     out = b.slab.view("_update", i).view(G.shape)
                     blocks = split_blocks(p.shape, max_dim) if merging and group.get("split") and p.dim() > 0 else None
                     if blocks is None:
-                        if precondition(self._state0(p), G0, G, out, int(b.slab.offsets_np[i])):
+                        if precondition(self._state0(p), G0, G, out, int(b.slab.offsets_np[i]), gdt):
                             updated.append(i)
                         continue
                     # split: every block is preconditioned on its own, with its own state (heavyball/utils.py:274-286, :1612-1623);
@@ -397,7 +433,7 @@ class SOAP(HBOptimizer):
                         g0b = G0[where].contiguous().reshape(bshape)
                         gb = g0b if G is G0 else G[where].contiguous().reshape(bshape)
                         ob = torch.empty_like(gb)
-                        if precondition(self.state[p].setdefault(k, {}), g0b, gb, ob, start):
+                        if precondition(self.state[p].setdefault(k, {}), g0b, gb, ob, start, gdt):
                             out[where].copy_(ob.reshape(out[where].shape))
                             done = True
                         start += gb.numel()
@@ -405,9 +441,10 @@ class SOAP(HBOptimizer):
                         updated.append(i)
                 if refresh:
                     self._refresh(gemm, refresh)
-                    for job in refresh:
-                        if len(job) > 3:
-                            self._narrow(L, job[3], K_M, job[2], mom_fmt, _lib.STREAM_SOAP_ROTATE, step, job[4], stream)
+                    for GG32, Q32, exp_avg, st, base in refresh:
+                        if mom_fmt != _lib.FMT_F32:
+                            self._narrow(L, st, K_M, exp_avg, mom_fmt, _lib.STREAM_SOAP_ROTATE, step, base, stream)
+                        self._store_factors(L, st, K_Q, Q32, _lib.STREAM_SOAP_Q, step, base, stream)  # heavyball/utils.py:898-900
             if updated:
                 pending.append((b, sorted(updated), items, keep))
         # tensors that split cuts up: their per-tensor update clip and caution's count are per block (torch on block views)
@@ -501,11 +538,33 @@ class SOAP(HBOptimizer):
                     for key in (K_M, K_V, K_M + "::ecc", K_V + "::ecc"):
                         if isinstance(st.get(key), torch.Tensor):
                             st[key] = st[key].to(self._role_dtype(group, key), copy=True).contiguous()
-                    for key in (K_Q, K_GG):
+                    for key in (K_Q, K_GG):  # in the dtype they come back in: torch's load has cast them to the parameter's
                         if isinstance(st.get(key), (list, tuple)):
-                            st[key] = [None if t is None else t.to(torch.float32, copy=True).contiguous() for t in st[key]]
+                            st[key] = [None if t is None else t.to(t.dtype if t.dtype in _PLAIN_FMT else torch.float32, copy=True).contiguous()
+                                       for t in st[key]]  # fmt: skip
 
     # -- pieces ----------------------------------------------------------------------------------------------------
+    @staticmethod
+    def _factors32(st):
+        """The factors and bases of a state as the fp32 tensors the products run on: the stored ones, or - kept in a 16-bit
+        dtype - fp32 copies of them for the length of the step."""
+        widen = lambda ts: [t if t is None or t.dtype == torch.float32 else t.float() for t in ts]  # noqa: E731
+        return widen(st[K_GG]), widen(st[K_Q])
+
+    def _store_factors(self, L, st, key, values32, stream_id, step, base, stream):
+        """``copy_stochastic_`` of freshly computed fp32 factors or bases into their 16-bit storage (heavyball/utils.py:1048,
+        :898-900), side li with noise stream ``stream_id + 2 * li`` at the places ``base + e``; the fp32 copies then take the
+        stored values again.  Nothing to do for fp32 storage, where ``values32`` are the stored tensors."""
+        for li, (t, v) in enumerate(zip(st[key], values32)):
+            if t is None or t is v:
+                continue
+            if t.dtype == torch.bfloat16:
+                _lib.check(L.hb_sr_bf16(v.data_ptr(), t.data_ptr(), t.numel(), self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF,
+                                        stream_id + 2 * li, base, stream), "hb_sr_bf16")  # fmt: skip
+            else:
+                t.copy_(v)
+            v.copy_(t)
+
     def _widen(self, L, st, key, fmt, stream):
         """The moment ``st[key]`` as fp32: itself when stored so, else a decoded copy."""
         t = st[key]

@@ -105,6 +105,8 @@ enum {
   HB_STREAM_SOAP_ROTATE = 11, /* SOAP: exp_avg written back to bf16 / ECC storage after its rotation into a refreshed basis */
   HB_STREAM_UPDATE_CLIP = 12, /* bf16 stochastic rounding of a clipped bf16 update (update_clipping with bf16 gradients); its own
                                  stream, so that a step with both clips draws independent noise for the two roundings */
+  HB_STREAM_SOAP_GG = 16,     /* SOAP under 16-bit gradients: a factor kept in bf16, rewritten after its update; side li draws from 16 + 2 li */
+  HB_STREAM_SOAP_Q = 17,      /* ... and a refreshed eigenbasis kept in bf16: 17 + 2 li */
 };
 
 /*

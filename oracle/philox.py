@@ -44,6 +44,8 @@ STREAM_EXP_AVG_SLOW = 9  # ECC / SR write of AdEMAMix's slow momentum
 STREAM_UPDATE = 10  # rounding of an un-fused transform's update into a 16-bit update buffer (update clipping)
 STREAM_SOAP_ROTATE = 11  # ECC / SR write of SOAP's exp_avg after its rotation into a refreshed eigenbasis
 STREAM_UPDATE_CLIP = 12  # bf16 stochastic rounding of a clipped bf16 update (independent of STREAM_CLIP, the gradient clip's)
+STREAM_SOAP_GG = 16  # SR write of a SOAP factor kept in bf16 (16-bit gradients): 16 + 2 * side
+STREAM_SOAP_Q = 17  # SR write of a refreshed SOAP eigenbasis kept in bf16: 17 + 2 * side
 
 
 def philox4x32_10(c0, c1, c2, c3, k0, k1):

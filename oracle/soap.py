@@ -79,8 +79,23 @@ def dim_merger(t: Tensor, max_precond_dim: int, split: bool):
     return out
 
 
-def update_ggt(grad: Tensor, GG: List[Optional[Tensor]], max_precond_dim: int, precondition_1d: bool, beta):
-    """heavyball/utils.py:1205-1221: GG_i <- GG_i * (1 - a) + (contraction of grad with itself over all but dim i) * a, a = 1 - beta."""
+def side_noise_index(tidx, n: int):
+    """The tensor index handed to the rounding for a factor or a basis of n elements that belongs to (the block of) a parameter:
+    element e takes the noise of place ``start + e`` of the parameter, ``start`` being where the block's own moments start."""
+    if isinstance(tidx, tuple):
+        return (tidx[0], np.uint64(tidx[1][0] if len(tidx[1]) else 0) + np.arange(n, dtype=np.uint64))
+    return (tidx, np.arange(n, dtype=np.uint64))
+
+
+def update_ggt(grad: Tensor, GG: List[Optional[Tensor]], max_precond_dim: int, precondition_1d: bool, beta, rounding=None, tidx=0):
+    """heavyball/utils.py:1205-1221: GG_i <- GG_i * (1 - a) + (contraction of grad with itself over all but dim i) * a, a = 1 - beta.
+    A factor kept in a 16-bit dtype (it has the dtype of the gradient it was created from, :1381) is rewritten through
+    copy_stochastic_ (:1048); the contraction runs in the dtype of ``grad`` as handed over: the gradient's own on the first step
+    (:1387), fp32 afterwards (heavyball/chainable.py:1248)."""
+    from . import first_order as fo
+    from . import philox
+    from .rounding import HalfRounding
+
     if grad.dim() == 2 and (not precondition_1d or grad.shape[1] > max_precond_dim):
         return
     g0 = einsum_base[: grad.dim() - 1]
@@ -92,18 +107,26 @@ def update_ggt(grad: Tensor, GG: List[Optional[Tensor]], max_precond_dim: int, p
         outer = torch.einsum(f"...{g0},...{g1}->...{b + b.upper()}", grad, grad)
         a = 1 - beta
         a = a.to(torch.float32) if isinstance(a, Tensor) else f32(a)
-        m.copy_(m * (1 - a) + outer * a)  # stochastic_lerp_ on fp32 (heavyball/utils.py:1048)
+        if m.dtype == torch.float32:
+            m.copy_(m * (1 - a) + outer * a)  # stochastic_lerp_ on fp32 (heavyball/utils.py:1048)
+        else:
+            fo.copy_stochastic(m, fo.promote(m) * (1 - a) + fo.promote(outer) * a, rounding or HalfRounding(), philox.STREAM_SOAP_GG + 2 * idx,
+                               side_noise_index(tidx, m.numel()))  # fmt: skip
 
 
 def symmetric_basis(m: Tensor, min_eps=1e-30) -> Tensor:
     """heavyball/utils.py:986-1003 on the path that does not raise: eigh(m + eps I), eigenvectors in descending order."""
-    eye = torch.eye(m.shape[-1], dtype=m.dtype)
-    _, vec = torch.linalg.eigh(m + min_eps * eye)
-    return torch.flip(vec, [-1]).contiguous()
+    from . import first_order as fo
+
+    m32 = fo.promote(m)  # :992; the basis goes back to the factor's dtype (:996, :1003)
+    eye = torch.eye(m32.shape[-1], dtype=m32.dtype)
+    _, vec = torch.linalg.eigh(m32 + min_eps * eye)
+    return torch.flip(vec, [-1]).contiguous().to(m.dtype)
 
 
-def init_preconditioner(grad: Tensor, max_precond_dim: int, precondition_1d: bool):
-    """heavyball/utils.py:1362-1388 with init_factor = 0; ``grad`` carries the bucket dimension."""
+def init_preconditioner(grad: Tensor, max_precond_dim: int, precondition_1d: bool, rounding=None, tidx=0):
+    """heavyball/utils.py:1362-1388 with init_factor = 0; ``grad`` carries the bucket dimension.  Factors and bases take the
+    gradient's dtype."""
     GG: List[Optional[Tensor]] = []
     if grad.numel() > 1 and (grad.ndim > 2 or precondition_1d):
         n = grad.shape[0]
@@ -114,7 +137,7 @@ def init_preconditioner(grad: Tensor, max_precond_dim: int, precondition_1d: boo
                 GG.append(torch.zeros(n, sh, sh, dtype=grad.dtype))
     else:
         GG.append(None)
-    update_ggt(grad, GG, max_precond_dim, precondition_1d, 0)
+    update_ggt(grad, GG, max_precond_dim, precondition_1d, 0, rounding, tidx)
     Q = [None if m is None else symmetric_basis(m) for m in GG]
     return GG, Q
 
@@ -125,7 +148,9 @@ def project(grad: Tensor, Q: List[Optional[Tensor]], back: bool) -> Tensor:
     pre = ",".join(["..." + (g + g.upper())[:: -1 if back else 1] for m, g in zip(Q, param) if m is not None])
     if pre:
         out = "".join([c.upper() if c.upper() in pre else c for c in param])
-        grad = torch.einsum(f"...{param},{pre}->...{out}", grad, *[q for q in Q if q is not None]).to(grad.dtype)
+        from . import first_order as fo
+
+        grad = torch.einsum(f"...{param},{pre}->...{out}", fo.promote(grad), *[fo.promote(q) for q in Q if q is not None]).to(grad.dtype)
     return grad
 
 
@@ -167,6 +192,7 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
         if m is None:
             new_qs.append(None)
             continue
+        m, q = fo.promote(m), fo.promote(q)  # heavyball/utils.py:850, :857
         tmp = m @ q
         eig = torch.einsum("...ij,...ij->...j", q, tmp)
         if eig.shape[-1] > 1:
@@ -183,11 +209,15 @@ def refresh_basis(GG: List[Optional[Tensor]], Q: List[Optional[Tensor]], exp_avg
     to_sh = ",".join([f"...{i}{o}" for m, i, o in zip(new_qs, in_str.upper(), out_str) if m is not None])
     out_lin = "".join([o if o in to_sh else i for i, o in zip(in_str, out_str)])
     subs = f"...{in_str},{from_sh},{to_sh}->...{out_lin}"
-    rotated = torch.einsum(subs, exp_avg, *[q for q in Q if q is not None], *[q for q in new_qs if q is not None])
+    rotated = torch.einsum(subs, exp_avg, *[fo.promote(q) for q in Q if q is not None], *[q for q in new_qs if q is not None])
     fo.copy_stochastic(stored, rotated, rounding or HalfRounding(), philox.STREAM_SOAP_ROTATE, tidx)
-    for q, qn in zip(Q, new_qs):
-        if q is not None:
+    for li, (q, qn) in enumerate(zip(Q, new_qs)):
+        if q is None:
+            continue
+        if q.dtype == torch.float32:
             q.copy_(qn)
+        else:  # heavyball/utils.py:898-900: the new basis into a 16-bit one through copy_stochastic_
+            fo.copy_stochastic(q, qn, rounding or HalfRounding(), philox.STREAM_SOAP_Q + 2 * li, side_noise_index(tidx, q.numel()))
     return key_gap
 
 
@@ -321,9 +351,14 @@ class SOAPOracle:
 
             fn = {"l2_clip_": fo.l2_clip, "rmsnorm_clip_": fo.rmsnorm_clip, "global_l2norm_clip": fo.global_l2norm_clip,
                   "global_rmsnorm_clip": fo.global_rmsnorm_clip}[self.gradient_clipping]  # fmt: skip
-            views = [u for k in updates for u in self._views(updates[k])]  # under split the norms are per block
-            for u, c in zip(views, fn(views)):
-                u.copy_(c.to(u.dtype))
+            from . import philox
+
+            views, tix = [], []  # under split the norms are per block
+            for k in updates:
+                views += self._views(updates[k])
+                tix += self._noise_index(k, updates[k].shape)
+            for u, c, t in zip(views, fn(views), tix):  # heavyball/utils.py:3226-3232 writes back through copy_stochastic_
+                fo.copy_stochastic(u, c, self.rounding.at_step(int(step)), philox.STREAM_CLIP, t)
         for i, (p, g) in enumerate(zip(self.params, grads)):
             if g is None:
                 continue
@@ -333,22 +368,25 @@ class SOAPOracle:
             shared = self._noise_index(i, g.shape)
             for k, (p, g, upd) in enumerate(blocks):
                 st = self._block_state(i, k)
-                u = upd.reshape(self._view_shape(g.shape)).unsqueeze(0)  # merged view + the bucket dimension
+                from . import first_order as fo
+
+                # merged view + the bucket dimension; the preconditioner promotes what it is handed (heavyball/chainable.py:1261, :1248)
+                u = fo.promote(upd).reshape(self._view_shape(g.shape)).unsqueeze(0)
+                rounding = self.rounding.at_step(int(step))
                 if self.K_M not in st:  # first step: ZeroGuard + GeneralGuard init, no update (heavyball/chainable.py:372-377)
                     self._moment(st, self.K_M, u)
                     self._moment(st, self.K_V, u)
                     # heavyball/chainable.py:1235-1238: the initial factors come from the gradient, not from the (clipped) update
                     g0 = g.clone().reshape(self._view_shape(g.shape)).unsqueeze(0)
-                    st[self.K_GG], st[self.K_Q] = init_preconditioner(g0, self.max_precond_dim, self.precondition_1d)
+                    st[self.K_GG], st[self.K_Q] = init_preconditioner(g0, self.max_precond_dim, self.precondition_1d, rounding, private[k])
                     continue
                 Q, GG = st[self.K_Q], st[self.K_GG]
                 gp = project(u, Q, False)
-                rounding = self.rounding.at_step(int(step))
                 m_st, v_st = self._moment(st, self.K_M, u), self._moment(st, self.K_V, u)
                 precond = adam_(m_st, v_st, gp, self.betas[0], self.betas[1], step - 1, self.eps, rounding, private[k])
                 precond = project(precond, Q, True)
                 beta = beta_debias(self.shampoo_beta, step)  # heavyball/chainable.py:1244
-                update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta)
+                update_ggt(u, GG, self.max_precond_dim, self.precondition_1d, beta, rounding, private[k])
                 if is_precond:
                     gap = refresh_basis(GG, Q, m_st, rounding, private[k])
                     self.sort_key_gap[(i, k)] = min(self.sort_key_gap.get((i, k), 1.0), gap)

@@ -195,7 +195,7 @@ def make_ecc():
 
 
 # ------------------------------------------------------------------------------------------------------
-def run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale=1e-2, param_scale=0.02, none_grad_for=None, mode=None):
+def run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale=1e-2, param_scale=0.02, none_grad_for=None, mode=None, param_dtype=None):
     if mode is not None:  # heavyball.utils.zeroth_power_mode for the length of the run, recorded as meta/zeroth_power_mode
         before, heavyball.utils.zeroth_power_mode = heavyball.utils.zeroth_power_mode, mode
         try:
@@ -208,7 +208,7 @@ def run_traj(name, cls, kwargs, shapes, grad_dtype, steps, grad_scale=1e-2, para
         torch.save(out, path)
         return
     gen = torch.Generator().manual_seed(0)
-    params = [torch.nn.Parameter(torch.randn(s, generator=gen) * param_scale) for s in shapes]
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * param_scale).to(param_dtype or torch.float32)) for s in shapes]
     for p in params:
         p.grad_dtype = None  # torch >= 2.9 refuses a gradient of another dtype otherwise
     out = {"meta/name": name, "meta/kwargs": json.dumps(kwargs), "meta/cls": cls.__name__, "meta/steps": steps}
@@ -391,6 +391,20 @@ def make_soap_split_combinations():
              torch.float32, 6)  # fmt: skip
 
 
+def make_soap_narrow_gradients():
+    """SOAP under 16-bit gradients without promote: the preconditioner promotes its input (heavyball/chainable.py:1261), but the
+    factors and the eigenbases are created in the gradient's dtype (heavyball/utils.py:1381, :996), the factors are rewritten
+    through copy_stochastic_ at every step and the bases at every refresh."""
+    shapes = [(8, 16), (16,), (12, 6)]
+    run_traj("soap_bf16grad", heavyball.SOAP, dict(precondition_frequency=3), shapes, torch.bfloat16, 6)
+    run_traj("soap_fp16grad_caution", heavyball.SOAP, dict(precondition_frequency=3, caution=True), shapes, torch.float16, 6)
+    run_traj("soap_bf16grad_mars_clip_l2", heavyball.SOAP, dict(precondition_frequency=3, mars=True, mars_gamma=0.1, gradient_clipping="l2_clip_"),
+             shapes, torch.bfloat16, 6, grad_scale=1.0)  # fmt: skip
+    run_traj("soap_bf16param", heavyball.SOAP, dict(precondition_frequency=3, weight_decay=0.1), shapes, torch.bfloat16, 6, param_dtype=torch.bfloat16)
+    run_traj("soap_bf16grad_split_ecc", heavyball.SOAP, dict(precondition_frequency=3, split=True, max_precond_dim=8, ecc="bf16+8"),
+             [(20, 12), (16,), (6, 30)], torch.bfloat16, 6)  # fmt: skip
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -548,7 +562,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "soapnarrow", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -575,6 +589,8 @@ if __name__ == "__main__":
         make_soap_mars_combinations()
     if "soapsplit" in which:
         make_soap_split_combinations()
+    if "soapnarrow" in which:
+        make_soap_narrow_gradients()
     if "switches" in which:
         make_more_switches()
     if "ns5" in which:
