@@ -22,7 +22,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(float x) {  // v_cvt_pk_bf16
   return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
 }
 __device__ __forceinline__ float f16_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
-__device__ __forceinline__ uint32_t f32_to_f16_rne(float x) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x); }
+// The empty asm makes x an fp32 value in a register first.  Without it the compiler folds a product or sum that feeds the
+// conversion into v_fma_mixlo_f16, which rounds the exact result once; the reference rounds to fp32, then to fp16 (torch computes
+// float16 tensors in fp32 and converts), and the two differ where the fp32 rounding lands on a float16 tie.
+__device__ __forceinline__ uint32_t f32_to_f16_rne_plain(float x) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x); }  // x is no product or sum
+__device__ __forceinline__ uint32_t f32_to_f16_rne(float x) {
+  asm("" : "+v"(x));
+  return f32_to_f16_rne_plain(x);
+}
 
 // ---------------------------------------------------------------------------------------------------------
 // Philox4x32-10 (Salmon et al., SC'11).  One call yields 128 bits: 16 bits for each of the 4 elements of a quartet

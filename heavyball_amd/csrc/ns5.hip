@@ -51,7 +51,7 @@ struct Problem {
   int tiles_m, tiles_n;              // tile grid of C
   int pos_begin;                     // where this run starts in the tile list of its XCD
   int t0, n_run;                     // the run: tiles t0 .. t0 + n_run - 1 of the matrix' tile list
-  int round_out;  // ModeFinal: the reference's update buffer is bf16, so the scaled result is rounded to bf16 (to nearest)
+  int round_out;  // ModeFinal: the reference's update buffer is 16 bits wide (1 bf16, 2 fp16): cast and scaling round to it (to nearest)
 };
 static_assert(sizeof(Problem) % 16 == 0, "tables of problems are moved in 16-byte pieces");
 // A table: this header, then the entries of XCD 0, of XCD 1, ...; entries [first[x], first[x + 1]) are XCD x's, in list order
@@ -259,7 +259,9 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
               o[r] = acc[i][j][rb4 * 4 + r];  // one K chunk of a split product: summed and rounded by ns_split_reduce_kernel
             } else {
               o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
-              if (g.round_out) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
+              if (g.round_out == 1) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
+              else if (g.round_out == 2)  // fp16: the cast leaves bf16's range (subnormals, overflow), then the product rounds again
+                o[r] = f16_to_f32(f32_to_f16_rne(f16_to_f32(f32_to_f16_rne(bf16_to_f32(prim[rb4 * 4 + r]))) * g.scale));
             }
           }
           if (g.f_transposed) {
@@ -640,7 +642,9 @@ struct PrepItem {
   int n_blocks, block_begin;  // sum of squares: this matrix owns workgroups [block_begin, block_begin + n_blocks)
   int tiles_c, tile_begin;    // conversion: 64 x 64 tiles, tiles_c per tile row, first workgroup id
   int legacy;                 // two stochastic rounds (legacy_zeropower_via_newtonschulz5) instead of one
-  int bf16_update;  // the reference's update buffer is bf16: norm and quotient are bf16 values (to nearest), no stochastic round
+  // the reference's update buffer is 16 bits wide.  1 (bf16): norm and quotient are bf16 values (to nearest), no stochastic round.
+  // 2 (fp16): norm and quotient are fp16 values (to nearest), the quotient is then rounded stochastically to bf16.
+  int narrow_update;
 };
 constexpr int kMaxPrep = 28;
 struct PrepGroup {
@@ -693,9 +697,14 @@ __global__ __launch_bounds__(256) void ns_norm_final_kernel(const PrepGroup grp)
   if (threadIdx.x == 0) {
     float nrm = __builtin_sqrtf((float)(lds[0] + lds[1] + lds[2] + lds[3]));
     float eps = grp.eps;
-    if (ka->it[pi].bf16_update) {  // a bf16 tensor's norm is a bf16 value; so is the clamp bound, except under the legacy schedule, whose
-      nrm = bf16_to_f32(f32_to_bf16_rne(nrm));  // division promotes both sides to fp32 first (heavyball/utils.py:1174-1179, :1190)
+    // a 16-bit tensor's norm is a value of its dtype; so is the clamp bound, except under the legacy schedule, whose division
+    // promotes both sides to fp32 first (heavyball/utils.py:1174-1179, :1190)
+    if (ka->it[pi].narrow_update == 1) {
+      nrm = bf16_to_f32(f32_to_bf16_rne(nrm));
       if (!ka->it[pi].legacy) eps = bf16_to_f32(f32_to_bf16_rne(eps));
+    } else if (ka->it[pi].narrow_update == 2) {
+      nrm = f16_to_f32(f32_to_f16_rne(nrm));  // infinite past 65504: the quotient is then zero, as in the reference
+      if (!ka->it[pi].legacy) eps = f16_to_f32(f32_to_f16_rne(eps));
     }
     ka->it[pi].norm[0] = __builtin_fmaxf(nrm, eps);  // G.norm().clamp(min=eps), heavyball/utils.py:555
   }
@@ -718,6 +727,7 @@ __device__ __forceinline__ uint32_t ns_round_one(float v, float nrm, int legacy,
     if (aligned) r = aligned[0];
     else r = rng.octet(flat & ~int64_t(7), HB_STREAM_NS_INPUT);
     if (legacy == 0) return sr_bf16(v / nrm, r.bits16(lane8));
+    if (legacy == 4) return sr_bf16(f16_to_f32(f32_to_f16_rne_plain(v / nrm)), r.bits16(lane8));  // fp16 update buffer: an fp16 quotient
   }
   if (aligned) r2 = aligned[1];
   else r2 = rng.octet(flat & ~int64_t(7), HB_STREAM_NS_INPUT + 1);
@@ -734,8 +744,10 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
   const float* __restrict__ g = ka->it[pi].g;
   const int rows = ka->it[pi].rows, cols = ka->it[pi].cols, transpose = ka->it[pi].transpose;
   const int64_t flat_base = ka->it[pi].flat_base;
-  // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input), 3: bf16 input under the legacy schedule (one, after the division)
-  const int legacy = ka->it[pi].bf16_update ? (ka->it[pi].legacy ? 3 : 2) : ka->it[pi].legacy;
+  // 0: one stochastic round, 1: two (legacy), 2: none (bf16 input), 3: bf16 input under the legacy schedule (one, after the division),
+  // 4: fp16 input, one round of the fp16 quotient (under the legacy schedule fp16 input takes 1: only its norm differs)
+  const int nu = ka->it[pi].narrow_update;
+  const int legacy = nu == 1 ? (ka->it[pi].legacy ? 3 : 2) : nu == 2 && !ka->it[pi].legacy ? 4 : ka->it[pi].legacy;
   const Rng rng = grp.rng;
   __shared__ uint16_t tile[64][64 + 8];  // +8: rows 144 B apart, so the column reads below spread over the banks
   const float nrm = ka->it[pi].norm[0];
@@ -761,7 +773,7 @@ __global__ __launch_bounds__(256) void ns_prep_kernel(const PrepGroup grp) {
         const float4 a = *reinterpret_cast<const float4*>(g + f0), b = *reinterpret_cast<const float4*>(g + f0 + 4);
         const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
         Rand8 rr[2];
-        if (legacy < 2) rr[0] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT);
+        if (legacy < 2 || legacy == 4) rr[0] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT);
         if (legacy & 1) rr[1] = rng.octet(flat_base + f0, HB_STREAM_NS_INPUT + 1);
 #pragma unroll
         for (int e = 0; e < 8; ++e) h[e] = ns_round_one(v[e], nrm, legacy, rng, flat_base + f0 + e, rr);
@@ -1049,7 +1061,8 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
   auto flag_of = [&](int i) { return flags[per_matrix ? i : 0]; };
   auto coeff_of = [&](int i, int k) { return coeffs_host[(per_matrix ? (size_t)i * 15 : 0) + k]; };
   for (int i = 0; i < n_mats; ++i)
-    if (flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE)) return set_error(HB_EINVAL, "%s: unknown flag bits", who);
+    if ((flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) || (flag_of(i) & (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) == (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE))
+      return set_error(HB_EINVAL, "%s: unknown flag bits, or both update formats at once", who);
   for (int i = 0; i < n_mats; ++i) {
     if (!g[i] || !out[i]) return set_error(HB_EINVAL, "%s: null matrix pointer at %d", who, i);
     if (rows[i] <= 0 || cols[i] <= 0 || rows[i] > (1 << 20) || cols[i] > (1 << 20)) return set_error(HB_EINVAL, "%s: bad shape at %d", who, i);
@@ -1100,7 +1113,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
       q.ldxt = (int)p.mp;
       q.transpose = p.rows > p.cols;
       q.legacy = (flag_of(i) & HB_NS_LEGACY) != 0;
-      q.bf16_update = (flag_of(i) & HB_NS_BF16_UPDATE) != 0;
+      q.narrow_update = (flag_of(i) & HB_NS_BF16_UPDATE) ? 1 : (flag_of(i) & HB_NS_F16_UPDATE) ? 2 : 0;
       const int64_t n = p.rows * p.cols;
       q.n_blocks = (int)std::min<int64_t>(1024, (n + 4095) / 4096);
       q.block_begin = blocks;
@@ -1198,7 +1211,7 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         } else {
           q.F = out[i]; q.f_transposed = p.rows > p.cols; q.ldf = (int)p.cols; q.f_rows = (int)p.rows; q.f_cols = (int)p.cols;
           q.scale = post_scale[i];
-          q.round_out = (flag_of(i) & HB_NS_BF16_UPDATE) != 0;
+          q.round_out = (flag_of(i) & HB_NS_BF16_UPDATE) ? 1 : (flag_of(i) & HB_NS_F16_UPDATE) ? 2 : 0;
         }
         probs[k] = q;
       }

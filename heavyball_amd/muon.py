@@ -10,6 +10,7 @@ from . import _lib
 from .optim import FirstOrder, HBOptimizer, _ECC_DTYPES, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, f32, lerp_weights, mars_weights, use_default
 
 #: per-iteration (a, b, c) of zeropower_via_newtonschulz5 (heavyball/utils.py:561-567)
+_NS_UPDATE_FLAG = {torch.float32: 0, torch.bfloat16: _lib.NS_BF16_UPDATE, torch.float16: _lib.NS_F16_UPDATE}
 NS_COEFFS = (
     (4.0848, -6.8946, 2.9270),
     (3.9505, -6.3029, 2.6377),
@@ -175,10 +176,6 @@ class Muon(HBOptimizer):
                 if not g.is_contiguous() or g.data_ptr() % 16 or g.device != b.device:
                     g = g.to(b.device).clone(memory_format=torch.contiguous_format)
                 by_dtype.setdefault(g.dtype, []).append((i, g))
-            if set(by_dtype) - {torch.float32, torch.bfloat16}:
-                # a float16 update buffer is normalised in float16 by the reference's Newton-Schulz (heavyball/utils.py:555): the
-                # result then depends on how the device at hand accumulates a float16 norm, which no fixture pins
-                raise NotImplementedError("Muon: float16 gradients (promote=True lifts them to float32 first)")
             for lst in by_dtype.values():
                 lst.sort(key=lambda t: t[0])
             prepared.append((b, items, by_dtype))
@@ -220,9 +217,9 @@ class Muon(HBOptimizer):
                     raise NotImplementedError(f"zeroth_power_mode={mode!r}")
                 # every matrix of the bucket goes through Newton-Schulz in the same grouped launches; under the legacy mode the
                 # square ones take the legacy coefficient table and input rounding (heavyball/utils.py:790-795), the others the default
-                # with bf16 gradients the reference's update buffer is bf16 and Newton-Schulz normalises it in bf16
-                # (per matrix: a bucket may hold gradients of both dtypes)
-                ns_flags = {i: _lib.NS_BF16_UPDATE if gdt == torch.bfloat16 else 0 for gdt, lst in by_dtype.items() for i, _ in lst}
+                # with 16-bit gradients the reference's update buffer has their dtype and Newton-Schulz normalises it there
+                # (per matrix: a bucket may hold gradients of several dtypes)
+                ns_flags = {i: _NS_UPDATE_FLAG[gdt] for gdt, lst in by_dtype.items() for i, _ in lst}
                 mats = []
                 for i, p, _ in items:
                     if p.dim() < 2:
@@ -254,6 +251,11 @@ class Muon(HBOptimizer):
                     with torch.cuda.device(b.device):
                         _lib.check(L.hb_sr_bf16(wide.data_ptr(), narrow.data_ptr(), wide.numel(), self._rng_mode(), self.rng_seed,
                                                 int(step) & 0xFFFFFFFF, _lib.STREAM_UPDATE_CLIP, 0, current_stream_ptr(b.device)), "hb_sr_bf16")  # fmt: skip
+                # a float16 update buffer takes the clipped values through a plain cast (heavyball/utils.py:2348-2349); they stay in
+                # the fp32 role, every one of them a float16 number
+                for i, _ in by_dtype.get(torch.float16, ()):
+                    wide = b.slab.view("_update", i)
+                    wide.copy_(wide.to(torch.float16))
         for b, items, by_dtype in prepared:
             offsets, numel = b.slab.meta()
             stream = current_stream_ptr(b.device)
@@ -292,7 +294,7 @@ class MuonAdamW(Muon, FirstOrder):
     gradients that is the same arithmetic as the fused Adam step, so the vectors run on ``hb_fused_step`` under the
     state names of the un-fused transform.  bf16 gradients on the vector route take the step kernel's update-only mode,
     which rounds the update to bf16 as that buffer does, and ``hb_update_param`` after it (fp16 gradients likewise, with
-    casts for roundings); fp16 gradients of matrices raise NotImplementedError (``promote=True`` lifts them to fp32 first).
+    casts for roundings).
     State names and initialisation sets follow the reference's index walk with the route in place
     (``nesterov_ema_momentum_4`` with {2, 3, 4}, ``exp_avg_exp_avg_4`` under ``nesterov=False``; ``scale_by_adam_exp_avg_0`` /
     ``_exp_avg_sq_0`` with {0}; ``mars_mars_old_grad_6`` and a 6 in both sets under ``mars``).  ``ecc`` / ``storage_dtype`` apply

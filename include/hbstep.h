@@ -251,8 +251,12 @@ int hb_momentum(void* momentum, void* momentum_corr, int32_t momentum_fmt, float
  * :2348-2349, :577, :808-809).  g and out stay fp32 buffers (holding bf16-representable values in that case).  Both flags
  * together: the legacy variant's first round is then the identity and its division, done in fp32 against the bf16-rounded
  * norm, keeps its stochastic round (stream HB_STREAM_NS_INPUT + 1; heavyball/utils.py:641-645, :1174-1179).
+ * HB_NS_F16_UPDATE says that the update buffer is float16 (fp16 gradients): the norm, the clamp bound and the quotient are
+ * fp16 values rounded to nearest, the quotient then takes the stochastic round to bf16 like an fp32 one, and the result is
+ * cast to fp16 and scaled there (two roundings to nearest).  With HB_NS_LEGACY only the norm is an fp16 value (its division
+ * runs in fp32).  The two update flags exclude each other.
  */
-enum { HB_NS_LEGACY = 1, HB_NS_BF16_UPDATE = 2 };
+enum { HB_NS_LEGACY = 1, HB_NS_BF16_UPDATE = 2, HB_NS_F16_UPDATE = 4 };
 int hb_ns5_workspace_bytes(int64_t rows, int64_t cols, int64_t* bytes);
 int hb_ns5(const float* g, float* out, int64_t rows, int64_t cols, const float* coeffs_host, int32_t legacy, float eps,
            float post_scale, int32_t rng_mode, uint64_t seed, uint32_t step, int64_t flat_base, void* workspace,

@@ -405,6 +405,33 @@ def make_soap_narrow_gradients():
              [(20, 12), (16,), (6, 30)], torch.bfloat16, 6)  # fmt: skip
 
 
+def make_muon_fp16_gradients():
+    """Muon on float16 gradients without promote: the norm, its clamp and the quotient are float16 arithmetic ahead of the bf16
+    stochastic round (heavyball/utils.py:555-556), the orthogonalised update goes back to float16 (:577) and is scaled there."""
+    shapes = [(8, 16), (16,), (24, 8), (4, 3, 6)]
+    run_traj("muon_fp16grad", heavyball.Muon, dict(weight_decay=0.01), shapes, torch.float16, 4)
+    run_traj("muon_fp16grad_mars_caution", heavyball.Muon, dict(mars=True, caution=True), shapes, torch.float16, 4)
+    run_traj("muonadamw_fp16grad_caution", heavyball.MuonAdamW, dict(caution=True, weight_decay=0.01), shapes, torch.float16, 4)
+    run_traj("muon_legacy_fp16grad", heavyball.Muon, dict(), [(16, 16), (16,), (24, 8), (8, 8)], torch.float16, 4, mode="legacy_newtonschulz")
+    # clips around the float16 route: both write into a float16 buffer through a plain cast (heavyball/utils.py:2348-2349)
+    run_traj("muon_updclip_l2_fp16grad", heavyball.Muon, dict(update_clipping="l2_clip_", lr=0.02), shapes, torch.float16, 4)
+    run_traj("muonadamw_clip_l2_updclip_global_rms_fp16grad", heavyball.MuonAdamW,
+             dict(gradient_clipping="l2_clip_", update_clipping="global_rmsnorm_clip", lr=0.02), shapes, torch.float16, 4, grad_scale=1.0)
+    out = {}
+    gen = torch.Generator().manual_seed(13)
+    for name, shape in [("sq", (16, 16)), ("wide", (8, 32)), ("tall", (32, 8)), ("sq64", (64, 64))]:
+        G = (torch.randn(shape, generator=gen) * 1e-2).half()
+        out[f"{name}/G"] = G.clone()
+        with half_rounding():
+            out[f"{name}/ns5"] = heavyball.utils.zeropower_via_newtonschulz5(G.clone(), 5).clone()
+            if shape[0] == shape[1]:
+                out[f"{name}/legacy"] = heavyball.utils.legacy_zeropower_via_newtonschulz5(G.clone(), 5).clone()
+            tmp = G.clone()
+            heavyball.utils.inplace_orthogonal_(tmp, out=tmp, scale_mode="scale")
+            out[f"{name}/orthogonal_scaled"] = tmp.clone()
+    torch.save(out, os.path.join(HERE, "ns5_fp16.pt"))
+
+
 def make_more_switches():
     """Muon, MuonAdamW and SOAP under switches beyond their defaults: MARS ahead of the momentum / the preconditioner, clipping
     and ECC on MuonAdamW, SOAP's preconditioner schedule."""
@@ -562,7 +589,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "soapnarrow", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "soapnarrow", "muonfp16", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -599,6 +626,8 @@ if __name__ == "__main__":
         make_muon()
     if "legacy" in which:
         make_legacy()
+    if "muonfp16" in which:
+        make_muon_fp16_gradients()
     if "soap" in which:
         make_soap()
     if "ckpt" in which:

@@ -40,7 +40,7 @@ def run_ns5(G, legacy=False, rng_mode=_lib.RNG_HALF, seed=0, step=0, base=0, sca
     arr = (ctypes.c_float * 15)(*ns_coeff_array(coeffs))
     if scale is None:
         scale = max(1, rows / cols) ** 0.5
-    flags = int(legacy) | (_lib.NS_BF16_UPDATE if G.dtype == torch.bfloat16 else 0)
+    flags = int(legacy) | {torch.bfloat16: _lib.NS_BF16_UPDATE, torch.float16: _lib.NS_F16_UPDATE}.get(G.dtype, 0)
     _lib.check(L.hb_ns5(g.data_ptr(), out.data_ptr(), rows, cols, arr, flags, 1e-7, scale, rng_mode, seed, step, base, ws.data_ptr(),
                         nbytes.value, None))
     torch.cuda.synchronize()
@@ -126,8 +126,24 @@ def test_ns5_mixed_schedules_in_one_call_equal_one_call_per_matrix():
         G = gs[k].cpu().bfloat16() if k in (1, 2, 6) else Gs[k]
         alone = run_ns5(G, legacy=legacy[k], rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=bases[k])
         assert torch.equal(outs[k].cpu().view(torch.int32), alone.view(torch.int32)), f"mixed update dtypes: matrix {k} {tuple(G.shape)}"
-    flags[0] |= 4  # an unknown flag bit is refused
-    assert L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None) != 0
+    # ... and HB_NS_F16_UPDATE: matrices 0 and 3 become float16 values beside the bf16 and fp32 ones
+    for k in (0, 3):
+        flags[k] |= _lib.NS_F16_UPDATE
+        gs[k].copy_(gs[k].half().float())
+    _lib.check(L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None))
+    torch.cuda.synchronize()
+    for k in (0, 3, 1, 7):
+        G = gs[k].cpu().half() if k in (0, 3) else gs[k].cpu().bfloat16() if k == 1 else Gs[k]
+        alone = run_ns5(G, legacy=legacy[k], rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=bases[k])
+        assert torch.equal(outs[k].cpu().view(torch.int32), alone.view(torch.int32)), f"three update dtypes: matrix {k} {tuple(G.shape)}"
+    call = lambda: L.hb_ns5_batched_mixed(n, gp, op, rows, cols, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 5, 3, base, ws.data_ptr(), nbytes.value, None)  # noqa: E731
+    flags[7] |= 8  # an unknown flag bit is refused
+    assert call() != 0
+    flags[7] &= ~8
+    assert call() == 0
+    flags[0] |= _lib.NS_BF16_UPDATE  # so are both update formats at once
+    assert call() != 0
+    torch.cuda.synchronize()
 
 
 def test_ns5_of_a_bucket_with_more_matrices_than_a_kernel_argument_holds():
@@ -217,6 +233,61 @@ def test_ns5_on_bf16_inputs_matches_reference_vectors(name):
     if f"{name}/legacy" in d:
         got = run_ns5(G, legacy=True, scale=1.0)
         assert torch.equal(got, got.bfloat16().float()) and rel_fro(got, d[f"{name}/legacy"].float()) < NS_TOL
+
+
+@pytest.mark.parametrize("name", ["sq", "wide", "tall", "sq64"])
+def test_ns5_on_fp16_inputs_matches_reference_vectors(name):
+    """HB_NS_F16_UPDATE, alone and with the legacy schedule, against vectors the reference computed on float16 tensors."""
+    d = torch.load(os.path.join(GOLDEN, "ns5_fp16.pt"), weights_only=True)
+    print("case", name, flush=True)
+    G = d[f"{name}/G"]
+    got = run_ns5(G, scale=1.0)
+    assert torch.equal(got, got.half().float()) and rel_fro(got, d[f"{name}/ns5"].float()) < NS_TOL
+    got = run_ns5(G)
+    assert torch.equal(got, got.half().float()) and rel_fro(got, d[f"{name}/orthogonal_scaled"].float()) < NS_TOL
+    if f"{name}/legacy" in d:
+        got = run_ns5(G, legacy=True, scale=1.0)
+        assert torch.equal(got, got.half().float()) and rel_fro(got, d[f"{name}/legacy"].float()) < NS_TOL
+
+
+@pytest.mark.parametrize("legacy", [False, True])
+def test_ns5_fp16_input_and_output_roundings_are_the_oracles(legacy):
+    """The float16 route through an identity schedule (a = 1, b = c = 0 makes an iteration return X): what comes back is the
+    normalised input after its roundings (float16 norm and quotient, one stochastic round to bf16; the legacy schedule rounds the
+    input first and divides in fp32) and the two roundings of the way out (the cast to float16, which flushes what bf16 still
+    resolves below 2^-24, and the scaling there).  Tiny entries make the cast lossy, the scale is not a power of two."""
+    from oracle import philox
+    from oracle.ecc import stochastic_round
+    gen = torch.Generator().manual_seed(3)
+    G = torch.randn(96, 160, generator=gen) * 1e-2
+    G[::3] *= 1e-5  # quotients below float16's normal range
+    G = G.half()
+    L = _lib.lib()
+    nbytes = ctypes.c_int64()
+    _lib.check(L.hb_ns5_workspace_bytes(96, 160, ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
+    g = G.to(DEV, torch.float32).contiguous()
+    out = torch.empty_like(g)
+    arr = (ctypes.c_float * 15)(*([1.0, 0.0, 0.0] * 5))
+    flags = int(legacy) | _lib.NS_F16_UPDATE
+    scale = 1.2345
+    print("case", legacy, flush=True)
+    _lib.check(L.hb_ns5(g.data_ptr(), out.data_ptr(), 96, 160, arr, flags, 1e-7, scale, _lib.RNG_PHILOX, 9, 4, 640, ws.data_ptr(), nbytes.value, None))
+    torch.cuda.synchronize()
+    nrm = G.norm()  # a float16 value
+    r = PhiloxRounding(9, step=4, base=[640])
+    if legacy:
+        x = stochastic_round(G.clone(), r.noise16(philox.STREAM_NS_INPUT, 0, G.shape))
+        x = stochastic_round(x.float() / nrm.float().clamp(min=1e-7), r.noise16(philox.STREAM_NS_INPUT + 1, 0, G.shape))
+    else:
+        x = stochastic_round(G / nrm.clamp(min=1e-7), r.noise16(philox.STREAM_NS_INPUT, 0, G.shape))
+    want = x.to(torch.float16)
+    want *= scale
+    got = out.cpu()
+    assert torch.equal(got, got.half().float())
+    want = want.float()
+    assert (got != want).float().mean() < 2e-3  # the norm's summation order may move its float16 rounding once in a while: then all differ
+    assert rel_fro(got, want) < 1e-2
 
 
 @pytest.mark.parametrize("legacy", [False, True])
@@ -323,6 +394,10 @@ MUON_VARIANTS = [
     # gradients of both dtypes in one bucket (dealt out in turn): the update buffer, and with it Newton-Schulz' normalisation, is per tensor
     ("mixed_grads", dict(lr=0.02, weight_decay=0.01), (torch.bfloat16, torch.float32)),
     ("mixed_grads_mars_ecc_caution", dict(lr=0.02, mars=True, ecc="bf16+8", caution=True), (torch.float32, torch.bfloat16)),
+    # float16 gradients: the update buffer is float16, Newton-Schulz normalises there and hands a float16 update back
+    ("fp16_grads", dict(lr=0.02, weight_decay=0.01), torch.float16),
+    ("fp16_grads_mars_caution_bf16_momentum", dict(lr=0.02, mars=True, caution=True, storage_dtype="bfloat16"), torch.float16),
+    ("three_grad_dtypes_ecc", dict(lr=0.02, ecc="bf16+16", weight_decay=0.01), (torch.float16, torch.bfloat16, torch.float32)),
 ]
 
 
@@ -379,7 +454,7 @@ def _random_muon_case(seed):
         kwargs["storage_dtype"] = "bfloat16"
     if rnd.random() < 0.3:
         kwargs["param_ecc"] = rnd.choice(["bf16+8", "bf16+16"])
-    gdt = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+    gdt = rnd.choice([torch.float32, torch.float32, torch.bfloat16, torch.float16])
     dims = [1, 2, 7, 8, 33, 64, 127, 128, 129, 200, 256, 300]
     shapes = [(rnd.choice(dims), rnd.choice(dims)) for _ in range(rnd.randint(2, 4))] + [(rnd.choice([1, 9, 64, 4097]),)]
     if rnd.random() < 0.4:

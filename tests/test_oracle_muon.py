@@ -49,6 +49,24 @@ def test_newton_schulz_on_bf16_inputs_matches_reference_vectors(name):
         assert out.dtype == torch.bfloat16 and rel_fro(out, d[f"{name}/legacy"]) < 1e-2
 
 
+@pytest.mark.parametrize("name", ["sq", "wide", "tall", "sq64"])
+def test_newton_schulz_on_fp16_inputs_matches_reference_vectors(name):
+    """A float16 update buffer: the norm and the quotient are float16 values, the quotient is rounded to bf16 like an fp32 one, the
+    result goes back to float16 and is scaled there (heavyball/utils.py:555-556, :577, :808-809).  Small matrices, whose products
+    are one block each: the oracle's arithmetic is the reference's, so the results are equal."""
+    d = torch.load(os.path.join(GOLDEN, "ns5_fp16.pt"), weights_only=True)
+    G = d[f"{name}/G"]
+    assert G.dtype == torch.float16
+    half = torch.full(G.shape, 1 << 15, dtype=torch.int32)
+    out = muon.newton_schulz5(G.clone(), half)
+    assert out.dtype == torch.float16 and torch.equal(out, d[f"{name}/ns5"])
+    if f"{name}/legacy" in d:
+        out = muon.legacy_newton_schulz5(G.clone(), half, half)
+        assert out.dtype == torch.float16 and torch.equal(out, d[f"{name}/legacy"])
+    out = muon.orthogonal(G.clone(), HalfRounding(), 0)
+    assert out.dtype == torch.float16 and torch.equal(out, d[f"{name}/orthogonal_scaled"])
+
+
 def test_polar_factor_invariant():
     """The per-iteration schedule drives every singular value towards 1: the result is close to U V^T of the SVD and
     its singular values lie in a band around 1 (a wrong coefficient, sign or a transposed operand leaves them far off)."""
