@@ -4,7 +4,8 @@ Per parameter (viewed with the reference's dimension merging, heavyball/utils.py
 the step is ``Ql^T G Qr`` -> Adam in the rotated basis -> ``Ql P Qr^T`` -> parameter update, plus the factor EMAs
 ``G G^T`` / ``G^T G``; a view that keeps more than two dimensions gets one rotation and one factor per dimension;
 every product runs on ``hb_gemm_f32``, the Adam part on ``hb_adam_precond``, the parameter update on ``hb_update_param``.
-The eigenbasis is initialised with ``torch.linalg.eigh`` on the first step (which performs no parameter update) and
+The eigenbasis is initialised on the first step (which performs no parameter update) with ``torch.linalg.eigh``, one solve
+per matrix on its smaller side with the other side's basis derived from it (``SOAP._first_bases``), and
 refreshed with one power-iteration step + a QR factorisation when the schedule fires (heavyball/utils.py:829-900,
 :986-1038, :3494-3500).  The QR runs on ``hb_orthonormalize_f32`` (block Gram-Schmidt on the GEMM kernel; its Q equals
 Householder's up to column signs, which the step is invariant to) and falls back to ``torch.linalg.qr`` when a factor is
@@ -361,20 +362,7 @@ class SOAP(HBOptimizer):
                             # 16-bit factors: the first one is the rounded product itself (the reference's contraction of a 16-bit
                             # gradient returns that dtype, utils.py:1387); the basis below comes from the stored values and is cast (:1003)
                             GG = [None if m is None else m.to(fdt) for m in GG]
-                        Q = []
-                        for m in GG:
-                            if m is None:
-                                Q.append(None)
-                                continue
-                            # heavyball/utils.py:1001-1003.  In float64: on a factor with a graded spectrum (singular values of
-                            # the gradient spread over two decades) the vendor's fp32 eigensolver leaves off-diagonal terms of
-                            # 1e-2 of the spectral norm in Q^T GG Q and the eigenvalues out of order, where LAPACK on the CPU,
-                            # which the reference's fixtures come from, leaves 4e-7; in float64 it leaves 1e-15, at
-                            # 0.7 s instead of 0.4 s for an 8192-wide factor, once.
-                            eye = torch.eye(m.shape[-1], dtype=torch.float64, device=m.device)
-                            _, vec = torch.linalg.eigh(m.double() + 1e-30 * eye)
-                            Q.append(torch.flip(vec, [-1]).to(fdt).contiguous())
-                        st[K_GG], st[K_Q] = GG, Q
+                        st[K_GG], st[K_Q] = GG, self._first_bases(G0, GG, fdt, base)
                         st.setdefault("is_initialized", set()).update({0, 2, 3})
                         return False
                     GG, Q = self._factors32(st)
@@ -616,6 +604,49 @@ class SOAP(HBOptimizer):
                 direct = out is not None and d == last and d in (0, X.dim() - 1)
                 cur = cls._mode_product(gemm, cur, q[0], d, back, out if direct else None)
         return cur
+
+    @staticmethod
+    def _eigh_basis(m: torch.Tensor) -> torch.Tensor:
+        """Eigenvectors of the symmetric ``m`` in float64, largest eigenvalue first (heavyball/utils.py:1001-1003).  In float64: on
+        a factor with a graded spectrum (singular values of the gradient spread over two decades) the vendor's fp32 eigensolver
+        leaves off-diagonal terms of 1e-2 of the spectral norm in Q^T GG Q and the eigenvalues out of order, where LAPACK on the
+        CPU, which the reference's fixtures come from, leaves 4e-7; in float64 it leaves 1e-15."""
+        eye = torch.eye(m.shape[-1], dtype=torch.float64, device=m.device)
+        _, vec = torch.linalg.eigh(m.double() + 1e-30 * eye)
+        return torch.flip(vec, [-1])
+
+    def _first_bases(self, G0, GG, fdt, seed_base: int):
+        """The eigenbases of the first factors (heavyball/utils.py:986-1038).
+
+        A matrix gradient G with both factors takes one eigensolve, on its smaller side: the first factors are G G^T and G^T G,
+        so the eigenvectors of one are the singular vectors of G on that side and the other side's follow as G^T U (or G U)
+        with normalised columns, in the same descending order.  Where the larger factor has more columns than G has rank, the
+        rest of its basis spans the null space of the factor, whose eigenvalues are rounding noise in any solver: any orthonormal
+        completion is an eigenbasis to that accuracy, and a seeded random one is taken.  ``hb_orthonormalize_f32`` then makes the
+        whole basis orthonormal to fp32 (its first columns already are, and stay).  An 8192-wide factor of a 2048 x 8192 gradient
+        costs 37 ms this way instead of a 670 ms eigensolve.  Everything else (factors kept in 16 bits, whose stored values are
+        no exact product any more; views with more than two dimensions; a single factor) takes the eigensolver per factor."""
+        Q: List[Optional[torch.Tensor]] = [None] * len(GG)
+        paired = fdt == torch.float32 and G0.dim() == 2 and len(GG) == 2 and GG[0] is not None and GG[1] is not None
+        done = set()
+        if paired:
+            s = 0 if G0.shape[0] <= G0.shape[1] else 1  # the smaller side
+            U = self._eigh_basis(GG[s][0])
+            W = (G0.T if s == 0 else G0).double() @ U  # [larger, smaller]: unnormalised singular vectors of the other side
+            norms = W.norm(dim=0)
+            good = norms > 1e-6 * norms.max()  # a column below that belongs to the null space of G itself
+            gen = torch.Generator(device=G0.device)
+            gen.manual_seed(0x50A9 + int(seed_base))  # the tensor's place in its slab: the same completion in every run
+            big, small = W.shape
+            other = torch.randn(big, big, device=G0.device, dtype=torch.float32, generator=gen)
+            other[:, :small] = torch.where(good, (W / norms.clamp(min=1e-300)).float(), other[:, :small])
+            if orthonormalize_(other):
+                Q[s], Q[1 - s] = U.to(fdt).contiguous()[None], other[None]
+                done = {0, 1}
+        for d, m in enumerate(GG):
+            if m is not None and d not in done:
+                Q[d] = self._eigh_basis(m).to(fdt).contiguous()
+        return Q
 
     @staticmethod
     def _update_ggt(gemm, G, GG, a: float, one_minus_a: float):

@@ -317,6 +317,61 @@ def test_soap_square_factors_own_eigh():
     _run_soap_vs_oracle([(40, 40), (24, 24)], dict(precondition_frequency=3), 7, 5e-3, adopt=False)
 
 
+@pytest.mark.parametrize("shape,kind", [((96, 512), "graded"), ((512, 96), "graded"), ((200, 200), "gauss"), ((64, 1024), "deficient"),
+                                        ((2048, 8192), "graded"), ((16, 8), "zero")])
+def test_soap_first_bases_from_one_eigensolve(shape, kind):
+    """The first step's bases of a matrix gradient: the smaller side's from eigh, the larger side's derived from it.  Both are
+    orthonormal, diagonalise the stored factors to fp32, list the eigenvalues in descending order (within the rounding noise that
+    fills the factor's null space), and the derived side's leading columns are, up to sign, the eigenvectors a solve on that side
+    finds.  "deficient": a gradient of rank 40, so the smaller factor has a null space of its own; "zero": a zero gradient."""
+    m, n = shape
+    gen = torch.Generator().manual_seed(m * 3 + n)
+    k = min(m, n)
+    if kind == "gauss":
+        G = torch.randn(m, n, generator=gen) * 1e-2
+    elif kind == "zero":
+        G = torch.zeros(m, n)
+    else:
+        u, _ = torch.linalg.qr(torch.randn(m, k, generator=gen, dtype=torch.float64))
+        v, _ = torch.linalg.qr(torch.randn(n, k, generator=gen, dtype=torch.float64))
+        sv = torch.logspace(0, -2, k, dtype=torch.float64)
+        if kind == "deficient":
+            sv[40:] = 0
+        G = ((u * sv) @ v.T * 1e-2).float()
+    print("case", shape, kind, flush=True)
+    G = G.to(DEV).contiguous()
+    p = torch.nn.Parameter(torch.zeros(m, n, device=DEV))
+    opt = heavyball_amd.SOAP([p], max_precond_dim=8192)
+    gemm = _Gemm(DEV)
+    GG = [torch.zeros(1, m, m, device=DEV), torch.zeros(1, n, n, device=DEV)]
+    opt._update_ggt(gemm, G, GG, 1.0, 0.0)
+    Q = opt._first_bases(G, GG, torch.float32, 0)
+    torch.cuda.synchronize()
+    assert [tuple(q.shape) for q in Q] == [(1, m, m), (1, n, n)] and all(q.dtype == torch.float32 and q.is_contiguous() for q in Q)
+    rank = {"deficient": 40, "zero": 0}.get(kind, k)
+    for q, gg in zip(Q, GG):
+        q, gg = q[0].double(), gg[0].double()
+        d = q.shape[0]
+        assert (q.T @ q - torch.eye(d, device=DEV, dtype=torch.float64)).abs().max().item() < 5e-6
+        D = q.T @ gg @ q
+        diag = D.diagonal()
+        top = diag.abs().max().item()
+        if kind == "zero":
+            assert top == 0
+            continue
+        assert (D - torch.diag(diag)).abs().max().item() < 1e-6 * top
+        assert (diag[1:] - diag[:-1]).max().item() < 1e-6 * top  # descending, up to the noise of the null space
+        assert diag[rank:].abs().max().item() < 1e-6 * top if rank < d else True
+        if kind != "gauss" and d <= 1024:  # eigenvalues two decades apart over d columns: the leading ones are well separated
+            _, vec = torch.linalg.eigh(gg)
+            lead = torch.flip(vec, [-1])[:, :8]
+            overlap = (lead * q[:, :8]).sum(0).abs()
+            assert overlap.min().item() > 0.999, overlap
+    # the same call again gives the same bases (the completion of the null space is seeded)
+    Q2 = opt._first_bases(G, GG, torch.float32, 0)
+    assert all(torch.equal(a, b) for a, b in zip(Q, Q2))
+
+
 def test_soap_mid_size_own_eigh_signed_momentum():
     """[256, 256] and [512, 512] Gaussian gradients with the optimizer's own eigh (no basis adopted) over two refreshes:
     square gradients give full-rank factors from the first step on, so the eigenbasis is unique up to column signs, and
