@@ -1049,17 +1049,18 @@ static size_t table_bytes(const std::vector<NsPlan>& plans) {
   return 20 * (8 * entries * sizeof(Problem) + 2 * (256 + sizeof(TableHeader)));
 }
 
-// coeffs_host: 15 floats per matrix when per_matrix, else one table of 15; flags likewise
-static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
+// coeffs_host: 3 * n_steps floats per matrix when per_matrix, else one table of that many; flags likewise
+static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols, int n_steps,
                             const float* coeffs_host, const int32_t* flags, bool per_matrix, float eps, const float* post_scale,
                             int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
                             int64_t workspace_bytes, hipStream_t s, const char* who) {
   if (n_mats <= 0 || !g || !out || !rows || !cols || !coeffs_host || !flags || !post_scale || !flat_base || !workspace)
     return set_error(HB_EINVAL, "%s: null pointer or empty batch", who);
   if (rng_mode != HB_RNG_HALF && rng_mode != HB_RNG_PHILOX) return set_error(HB_EINVAL, "%s: bad rng_mode", who);
+  if (n_steps < 1 || n_steps > 64) return set_error(HB_EINVAL, "%s: 1 to 64 iterations", who);
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return set_error(HB_EINVAL, "%s: workspace must be 256-byte aligned", who);
   auto flag_of = [&](int i) { return flags[per_matrix ? i : 0]; };
-  auto coeff_of = [&](int i, int k) { return coeffs_host[(per_matrix ? (size_t)i * 15 : 0) + k]; };
+  auto coeff_of = [&](int i, int k) { return coeffs_host[(per_matrix ? (size_t)i * 3 * n_steps : 0) + k]; };
   for (int i = 0; i < n_mats; ++i)
     if ((flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) || (flag_of(i) & (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) == (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE))
       return set_error(HB_EINVAL, "%s: unknown flag bits, or both update formats at once", who);
@@ -1131,95 +1132,101 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
     ns_prep_kernel<<<tiles, 256, 0, s>>>(pg);
   }
 
-  for (int cls = 0; cls < 2; ++cls) {
-    const int t = cls == 0 ? 256 : 128;
-    std::vector<int> idx;
-    for (int i = 0; i < n_mats; ++i)
-      if (tile[i] == t) idx.push_back(i);
-    if (idx.empty()) continue;
-    std::vector<Problem> probs(idx.size());
-    for (int it = 0; it < 5; ++it) {
-      const int cur = it & 1, nxt = cur ^ 1;
-      auto ca = [&](int i) { return coeff_of(i, 3 * it); };      // the iteration's (a, b, c) of matrix i
-      auto cb = [&](int i) { return coeff_of(i, 3 * it + 1); };
-      auto cc = [&](int i) { return coeff_of(i, 3 * it + 2); };
-      // S = X X^T, Y = c S + b I   (S is symmetric bit for bit: only the upper triangle of tiles is computed; a product
-      // that is split along K goes through raw partial products and ns_split_reduce_kernel instead)
-      std::vector<Problem> whole, chunks;
-      for (size_t k = 0; k < idx.size(); ++k) {
-        const int i = idx[k];
-        const NsPlan& p = plans[i];
-        Problem q{};
-        q.tiles_m = q.tiles_n = (int)(p.mp / t);
-        q.lda = (int)p.np; q.ldb = (int)p.np;
-        q.mul_c = cc(i); q.diag = cb(i);
-        if (p.split == 0) {
-          q.A = X(i, cur); q.B = X(i, cur); q.K = (int)p.np;
-          q.C = S(i); q.ldc = (int)p.mp; q.C2 = Y(i); q.ldc2 = (int)p.mp;
-          whole.push_back(q);
-          continue;
-        }
-        for (int c = 0; c < p.split; ++c) {
-          const int64_t k0 = (int64_t)c * p.split_chunk;
-          q.A = X(i, cur) + k0; q.B = X(i, cur) + k0;
-          q.K = (int)(p.np - k0 < p.split_chunk ? p.np - k0 : p.split_chunk);
-          q.F = reinterpret_cast<float*>(base[i] + p.off_split) + (size_t)c * p.mp * p.mp;
-          q.ldf = (int)p.mp; q.f_rows = (int)p.mp; q.f_cols = (int)p.mp; q.f_transposed = 0; q.scale = 1.0f;
-          chunks.push_back(q);
-        }
-      }
-      if (!whole.empty()) gemm_stage<kModeS>(st, whole, t, s);
-      if (!chunks.empty()) {
-        gemm_stage<kModePartial>(st, chunks, t, s);
+  // the tables in the workspace have room for five iterations: longer schedules run in groups of five, each group's tables
+  // written over the last one's (in stream order, behind the products that read those)
+  for (int it0 = 0; it0 < n_steps; it0 += 5) {
+    st = Stager();
+    for (int cls = 0; cls < 2; ++cls) {
+      const int t = cls == 0 ? 256 : 128;
+      std::vector<int> idx;
+      for (int i = 0; i < n_mats; ++i)
+        if (tile[i] == t) idx.push_back(i);
+      if (idx.empty()) continue;
+      std::vector<Problem> probs(idx.size());
+      for (int it = it0; it < std::min(it0 + 5, n_steps); ++it) {
+        const int cur = it & 1, nxt = cur ^ 1;
+        auto ca = [&](int i) { return coeff_of(i, 3 * it); };      // the iteration's (a, b, c) of matrix i
+        auto cb = [&](int i) { return coeff_of(i, 3 * it + 1); };
+        auto cc = [&](int i) { return coeff_of(i, 3 * it + 2); };
+        // S = X X^T, Y = c S + b I   (S is symmetric bit for bit: only the upper triangle of tiles is computed; a product
+        // that is split along K goes through raw partial products and ns_split_reduce_kernel instead)
+        std::vector<Problem> whole, chunks;
         for (size_t k = 0; k < idx.size(); ++k) {
           const int i = idx[k];
           const NsPlan& p = plans[i];
-          if (p.split == 0) continue;
-          const float* parts = reinterpret_cast<const float*>(base[i] + p.off_split);
-          uint16_t *s_out = S(i), *y_out = Y(i);
-          const float mul_c = cc(i), diag = cb(i);
-          const int split = p.split, mp = (int)p.mp;
-          st.ops.push_back([=](const char*) {
-            ns_split_reduce_kernel<<<(unsigned)((mp / 32) * (mp / 32)), 256, 0, s>>>(parts, split, mp, t, s_out, y_out, mul_c, diag);
-            return (int)HB_OK;
-          });
+          Problem q{};
+          q.tiles_m = q.tiles_n = (int)(p.mp / t);
+          q.lda = (int)p.np; q.ldb = (int)p.np;
+          q.mul_c = cc(i); q.diag = cb(i);
+          if (p.split == 0) {
+            q.A = X(i, cur); q.B = X(i, cur); q.K = (int)p.np;
+            q.C = S(i); q.ldc = (int)p.mp; q.C2 = Y(i); q.ldc2 = (int)p.mp;
+            whole.push_back(q);
+            continue;
+          }
+          for (int c = 0; c < p.split; ++c) {
+            const int64_t k0 = (int64_t)c * p.split_chunk;
+            q.A = X(i, cur) + k0; q.B = X(i, cur) + k0;
+            q.K = (int)(p.np - k0 < p.split_chunk ? p.np - k0 : p.split_chunk);
+            q.F = reinterpret_cast<float*>(base[i] + p.off_split) + (size_t)c * p.mp * p.mp;
+            q.ldf = (int)p.mp; q.f_rows = (int)p.mp; q.f_cols = (int)p.mp; q.f_transposed = 0; q.scale = 1.0f;
+            chunks.push_back(q);
+          }
         }
-      }
-      // Y2 = Y S + a I  (S symmetric: its rows are the K-contiguous operand; Y2 is a polynomial in S, so only the
-      // upper triangle of tiles is computed and mirrored)
-      for (size_t k = 0; k < idx.size(); ++k) {
-        const int i = idx[k];
-        const NsPlan& p = plans[i];
-        Problem q{};
-        q.A = Y(i); q.B = S(i); q.K = (int)p.mp; q.lda = (int)p.mp; q.ldb = (int)p.mp;
-        q.C = Y2(i); q.ldc = (int)p.mp;
-        q.tiles_m = q.tiles_n = (int)(p.mp / t);
-        q.diag = ca(i);
-        probs[k] = q;
-      }
-      gemm_stage<kModeY2>(st, probs, t, s);
-      // X = Y2 X  ==  gemm(Y2, X^T)
-      for (size_t k = 0; k < idx.size(); ++k) {
-        const int i = idx[k];
-        const NsPlan& p = plans[i];
-        Problem q{};
-        q.A = Y2(i); q.B = Xt(i, cur); q.K = (int)p.mp; q.lda = (int)p.mp; q.ldb = (int)p.mp;
-        q.tiles_m = (int)(p.mp / t);
-        q.tiles_n = (int)(p.np / t);
-        if (it < 4) {
-          q.C = X(i, nxt); q.ldc = (int)p.np; q.C2 = Xt(i, nxt); q.ldc2 = (int)p.mp;
-        } else {
-          q.F = out[i]; q.f_transposed = p.rows > p.cols; q.ldf = (int)p.cols; q.f_rows = (int)p.rows; q.f_cols = (int)p.cols;
-          q.scale = post_scale[i];
-          q.round_out = (flag_of(i) & HB_NS_BF16_UPDATE) ? 1 : (flag_of(i) & HB_NS_F16_UPDATE) ? 2 : 0;
+        if (!whole.empty()) gemm_stage<kModeS>(st, whole, t, s);
+        if (!chunks.empty()) {
+          gemm_stage<kModePartial>(st, chunks, t, s);
+          for (size_t k = 0; k < idx.size(); ++k) {
+            const int i = idx[k];
+            const NsPlan& p = plans[i];
+            if (p.split == 0) continue;
+            const float* parts = reinterpret_cast<const float*>(base[i] + p.off_split);
+            uint16_t *s_out = S(i), *y_out = Y(i);
+            const float mul_c = cc(i), diag = cb(i);
+            const int split = p.split, mp = (int)p.mp;
+            st.ops.push_back([=](const char*) {
+              ns_split_reduce_kernel<<<(unsigned)((mp / 32) * (mp / 32)), 256, 0, s>>>(parts, split, mp, t, s_out, y_out, mul_c, diag);
+              return (int)HB_OK;
+            });
+          }
         }
-        probs[k] = q;
+        // Y2 = Y S + a I  (S symmetric: its rows are the K-contiguous operand; Y2 is a polynomial in S, so only the
+        // upper triangle of tiles is computed and mirrored)
+        for (size_t k = 0; k < idx.size(); ++k) {
+          const int i = idx[k];
+          const NsPlan& p = plans[i];
+          Problem q{};
+          q.A = Y(i); q.B = S(i); q.K = (int)p.mp; q.lda = (int)p.mp; q.ldb = (int)p.mp;
+          q.C = Y2(i); q.ldc = (int)p.mp;
+          q.tiles_m = q.tiles_n = (int)(p.mp / t);
+          q.diag = ca(i);
+          probs[k] = q;
+        }
+        gemm_stage<kModeY2>(st, probs, t, s);
+        // X = Y2 X  ==  gemm(Y2, X^T)
+        for (size_t k = 0; k < idx.size(); ++k) {
+          const int i = idx[k];
+          const NsPlan& p = plans[i];
+          Problem q{};
+          q.A = Y2(i); q.B = Xt(i, cur); q.K = (int)p.mp; q.lda = (int)p.mp; q.ldb = (int)p.mp;
+          q.tiles_m = (int)(p.mp / t);
+          q.tiles_n = (int)(p.np / t);
+          if (it < n_steps - 1) {
+            q.C = X(i, nxt); q.ldc = (int)p.np; q.C2 = Xt(i, nxt); q.ldc2 = (int)p.mp;
+          } else {
+            q.F = out[i]; q.f_transposed = p.rows > p.cols; q.ldf = (int)p.cols; q.f_rows = (int)p.rows; q.f_cols = (int)p.cols;
+            q.scale = post_scale[i];
+            q.round_out = (flag_of(i) & HB_NS_BF16_UPDATE) ? 1 : (flag_of(i) & HB_NS_F16_UPDATE) ? 2 : 0;
+          }
+          probs[k] = q;
+        }
+        if (it < n_steps - 1) gemm_stage<kModeX>(st, probs, t, s);
+        else gemm_stage<kModeFinal>(st, probs, t, s);
       }
-      if (it < 4) gemm_stage<kModeX>(st, probs, t, s);
-      else gemm_stage<kModeFinal>(st, probs, t, s);
     }
+    if (int rc = run_staged(st, dev_tables, table_room, s, who)) return rc;
   }
-  return run_staged(st, dev_tables, table_room, s, who);
+  return HB_OK;
 }
 
 }  // namespace hb
@@ -1274,7 +1281,7 @@ extern "C" int hb_ns5_batched(int32_t n_mats, const float* const* g, float* cons
                               const float* coeffs_host, int32_t legacy, float eps, const float* post_scale, int32_t rng_mode,
                               uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                               void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, coeffs_host, &legacy, false, eps, post_scale, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, &legacy, false, eps, post_scale, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched");
 }
 
@@ -1282,13 +1289,21 @@ extern "C" int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float
                                     const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
                                     uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                                     void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, coeffs_host, flags, true, eps, post_scale, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, flags, true, eps, post_scale, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched_mixed");
+}
+
+extern "C" int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
+                                   int32_t n_steps, const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale,
+                                   int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
+                                   int64_t workspace_bytes, void* stream_) {
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, n_steps, coeffs_host, flags, true, eps, post_scale, rng_mode, seed, step, flat_base,
+                              workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns_batched_steps");
 }
 
 extern "C" int hb_ns5(const float* g, float* out, int64_t rows, int64_t cols, const float* coeffs_host, int32_t legacy, float eps,
                       float post_scale, int32_t rng_mode, uint64_t seed, uint32_t step, int64_t flat_base, void* workspace,
                       int64_t workspace_bytes, void* stream_) {
-  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, coeffs_host, &legacy, false, eps, &post_scale, rng_mode, seed, step, &flat_base, workspace,
+  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, 5, coeffs_host, &legacy, false, eps, &post_scale, rng_mode, seed, step, &flat_base, workspace,
                               workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5");
 }

@@ -9,8 +9,8 @@ import torch
 from . import _lib
 from .optim import FirstOrder, HBOptimizer, _ECC_DTYPES, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, f32, lerp_weights, mars_weights, use_default
 
-#: per-iteration (a, b, c) of zeropower_via_newtonschulz5 (heavyball/utils.py:561-567)
 _NS_UPDATE_FLAG = {torch.float32: 0, torch.bfloat16: _lib.NS_BF16_UPDATE, torch.float16: _lib.NS_F16_UPDATE}
+#: per-iteration (a, b, c) of zeropower_via_newtonschulz5 (heavyball/utils.py:561-567)
 NS_COEFFS = (
     (4.0848, -6.8946, 2.9270),
     (3.9505, -6.3029, 2.6377),
@@ -21,12 +21,25 @@ NS_COEFFS = (
 #: legacy_zeropower_via_newtonschulz5 (heavyball/utils.py:639)
 LEGACY_COEFFS = ((3.4445, -4.7750, 2.0315),) * 5
 
-#: module-level switch of the reference (heavyball/utils.py:25): "newtonschulz" or "legacy_newtonschulz"
+#: msign(x, 10) (heavyball/utils.py:587-602, :619): the polynomials of arXiv 2505.16932v3, all but the last divided by a safety
+#: factor (a / 1.01, b / 1.01^3, c / 1.01^5), the last one repeated to fill the ten steps
+_POLAR = (
+    (8.28721201814563, -23.595886519098837, 17.300387312530933),
+    (4.107059111542203, -2.9478499167379106, 0.5448431082926601),
+    (3.9486908534822946, -2.908902115962949, 0.5518191394370137),
+    (3.3184196573706015, -2.488488024314874, 0.51004894012372),
+    (2.300652019954817, -1.6689039845747493, 0.4188073119525673),
+    (1.891301407787398, -1.2679958271945868, 0.37680408948524835),
+    (1.8750014808534479, -1.2500016453999487, 0.3750001645474248),
+)
+POLAR_COEFFS = tuple((a / 1.01, b / 1.01**3, c / 1.01**5) for a, b, c in _POLAR) + ((1.875, -1.25, 0.375),) * 3
+
+#: module-level switch of the reference (heavyball/utils.py:25): "newtonschulz", "legacy_newtonschulz" or "thinky_polar_express"
 zeroth_power_mode = "newtonschulz"
 
 
 def ns_coefficients(coeffs) -> List[float]:
-    """The 15 floats ``hb_ns5`` takes, with the reference's CPU rounding of the scalars.
+    """The three floats per iteration that ``hb_ns5`` and its relatives take, with the reference's CPU rounding of the scalars.
 
     ``y = c * s`` multiplies the bf16 matrix by the scalar at fp32 precision, but ``y.diagonal().add_(b)`` is an in-place
     bf16 op whose scalar operand is first cast to the tensor's dtype (heavyball/utils.py:569-572 as executed by ATen on
@@ -213,10 +226,12 @@ class Muon(HBOptimizer):
                                              self._mom_mode, a_f, oma_f, self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF, stream),
                                "hb_momentum")  # fmt: skip
                 # orthogonalise every update with two or more dimensions (heavyball/chainable.py:1117-1126)
-                if mode not in ("newtonschulz", "legacy_newtonschulz"):
+                if mode not in ("newtonschulz", "legacy_newtonschulz", "thinky_polar_express"):
+                    # "qr", "svd", "legacy_svd" (heavyball/utils.py:798-806) are factorisations, not this iteration
                     raise NotImplementedError(f"zeroth_power_mode={mode!r}")
                 # every matrix of the bucket goes through Newton-Schulz in the same grouped launches; under the legacy mode the
-                # square ones take the legacy coefficient table and input rounding (heavyball/utils.py:790-795), the others the default
+                # square ones take the legacy coefficient table and input rounding (heavyball/utils.py:790-795), under
+                # "thinky_polar_express" the ten-step schedule of msign (:796-797, in a call of their own), the others the default
                 # with 16-bit gradients the reference's update buffer has their dtype and Newton-Schulz normalises it there
                 # (per matrix: a bucket may hold gradients of several dtypes)
                 ns_flags = {i: _NS_UPDATE_FLAG[gdt] for gdt, lst in by_dtype.items() for i, _ in lst}
@@ -226,8 +241,10 @@ class Muon(HBOptimizer):
                         continue
                     rows, cols = p.shape[0], p.numel() // p.shape[0]
                     mats.append((i, rows, cols))
-                coeff_tables = {False: ns_coefficients(NS_COEFFS), True: ns_coefficients(LEGACY_COEFFS)}
-                for part in self._ns_parts(L, mats):
+                coeff_tables = {False: ns_coefficients(NS_COEFFS), True: ns_coefficients(LEGACY_COEFFS), "polar": ns_coefficients(POLAR_COEFFS)}
+                polar = [m for m in mats if mode == "thinky_polar_express" and m[1] == m[2]]
+                plain = [m for m in mats if not (mode == "thinky_polar_express" and m[1] == m[2])]
+                for part, n_steps in [(q, 5) for q in self._ns_parts(L, plain)] + [(q, 10) for q in self._ns_parts(L, polar)]:
                     n = len(part)
                     legacy = [mode == "legacy_newtonschulz" and r == c for _, r, c in part]
                     rows_a = (ctypes.c_int64 * n)(*[r for _, r, _ in part])
@@ -235,13 +252,14 @@ class Muon(HBOptimizer):
                     ptrs = (ctypes.c_void_p * n)(*[b.slab.view("_update", i).data_ptr() for i, _, _ in part])
                     scale = (ctypes.c_float * n)(*[max(1, r / c) ** 0.5 for _, r, c in part])  # heavyball/utils.py:808-809
                     base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
-                    arr = (ctypes.c_float * (15 * n))(*[x for lg in legacy for x in coeff_tables[lg]])
+                    arr = (ctypes.c_float * (3 * n_steps * n))(*[x for lg in legacy for x in coeff_tables["polar" if n_steps == 10 else lg]])
                     flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) for (i, _, _), lg in zip(part, legacy)])
                     nbytes = ctypes.c_int64()
                     _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows_a, cols_a, ctypes.byref(nbytes)))
                     ws = self._ws(b.device, nbytes.value)
-                    _lib.check(L.hb_ns5_batched_mixed(n, ptrs, ptrs, rows_a, cols_a, arr, flag_a, 1e-7, scale, self._rng_mode(), self.rng_seed,
-                                                      int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream), "hb_ns5_batched_mixed")  # fmt: skip
+                    _lib.check(L.hb_ns_batched_steps(n, ptrs, ptrs, rows_a, cols_a, n_steps, arr, flag_a, 1e-7, scale, self._rng_mode(),
+                                                     self.rng_seed, int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream),
+                               "hb_ns_batched_steps")  # fmt: skip
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group
             keep.append((yield (self.update_clipping, "_update", [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared])))
             for b, items, by_dtype in prepared:

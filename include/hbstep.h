@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 9
+#define HB_ABI_VERSION 10
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -284,6 +284,16 @@ int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* ou
                          const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
                          uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                          void* stream);
+
+/* hb_ns5_batched_mixed with a schedule of n_steps iterations instead of five (coeffs_host: n_mats x 3 n_steps floats):
+ * replaces msign (heavyball/utils.py:605-631), the ten-step "Polar Express" schedule that square matrices take under
+ * zeroth_power_mode = "thinky_polar_express" (:796-797), followed by the same post-scale; normalisation, input rounding and
+ * the iteration are those of hb_ns5.  Same workspace as hb_ns5_batched for the same shapes; hb_ns5_batched_mixed is this call
+ * with n_steps = 5. */
+int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
+                        int32_t n_steps, const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale,
+                        int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
+                        int64_t workspace_bytes, void* stream);
 
 /* Test hook: ONE product of the Newton-Schulz iteration on bf16 operands (row-major, K contiguous: A [M, K], B [N, K]) through
  * the kernel of the given tile class (128 or 256), so that a test can put the same product through both kernels, whose

@@ -2,7 +2,7 @@
 oracle/__init__.py).
 
 Follows heavyball/utils.py:766-769 (``_compilable_nesterov_ema_``), :550-577 (``zeropower_via_newtonschulz5``),
-:637-657 (``legacy_zeropower_via_newtonschulz5``), :784-817 (``_compilable_orthogonal_``: which schedule runs and the
+:637-657 (``legacy_zeropower_via_newtonschulz5``), :605-631 (``msign``), :784-817 (``_compilable_orthogonal_``: which schedule runs and the
 ``max(1, rows/cols) ** 0.5`` post-scale) and heavyball/chainable.py:1117-1138 (``orthogonalize_update``, ``nesterov_ema``).
 
 bf16 matrix products call the same ATen op as the reference (``@`` on bf16 tensors): an fp32-accumulated product rounded
@@ -31,6 +31,20 @@ NS_COEFFS = (  # heavyball/utils.py:561-567
     (2.8366, -3.0525, 1.2012),
 )
 LEGACY_COEFFS = ((3.4445, -4.7750, 2.0315),) * 5  # heavyball/utils.py:639
+# heavyball/utils.py:587-602, :619: the published polynomials of arXiv 2505.16932v3, all but the last divided by a safety factor
+# (a / 1.01, b / 1.01^3, c / 1.01^5); a schedule longer than the table repeats its last entry.
+_POLAR = (
+    (8.28721201814563, -23.595886519098837, 17.300387312530933),
+    (4.107059111542203, -2.9478499167379106, 0.5448431082926601),
+    (3.9486908534822946, -2.908902115962949, 0.5518191394370137),
+    (3.3184196573706015, -2.488488024314874, 0.51004894012372),
+    (2.300652019954817, -1.6689039845747493, 0.4188073119525673),
+    (1.891301407787398, -1.2679958271945868, 0.37680408948524835),
+    (1.8750014808534479, -1.2500016453999487, 0.3750001645474248),
+    (1.875, -1.25, 0.375),
+)
+_POLAR_STABLE = tuple((a / 1.01, b / 1.01**3, c / 1.01**5) for a, b, c in _POLAR[:-1]) + (_POLAR[-1],)
+POLAR_COEFFS = tuple(_POLAR_STABLE[min(k, len(_POLAR_STABLE) - 1)] for k in range(10))  # msign(x, 10), heavyball/utils.py:796-797
 
 
 def bf16_matmul(a: Tensor, b: Tensor) -> Tensor:
@@ -63,6 +77,19 @@ def newton_schulz5(G: Tensor, noise16: Tensor, eps=1e-7) -> Tensor:
     return x.to(G.dtype)
 
 
+def polar_express(G: Tensor, noise16: Tensor, eps=1e-7) -> Tensor:
+    """heavyball/utils.py:605-631 (``msign`` with steps = 10): normalisation, input rounding and iteration of newton_schulz5 under
+    the ten-step schedule above."""
+    Gn = G / G.norm(dim=(-2, -1)).clamp(min=eps)
+    x = stochastic_round(Gn, noise16)
+    if G.size(-2) > G.size(-1):
+        x = x.mT
+    x = _iterate(x, POLAR_COEFFS)
+    if G.size(-2) > G.size(-1):
+        x = x.mT
+    return x.to(G.dtype)
+
+
 def legacy_newton_schulz5(G: Tensor, noise16_a: Tensor, noise16_b: Tensor, eps=1e-7) -> Tensor:
     """heavyball/utils.py:637-657: round to bf16 first, then divide by max(norm, eps) (a second stochastic round)."""
     x = stochastic_round(G.clone(), noise16_a)
@@ -79,6 +106,8 @@ def orthogonal(x: Tensor, rounding, tidx: int, mode="newtonschulz") -> Tensor:
     """heavyball/utils.py:784-817 with scale_mode="scale": non-square inputs always take the per-iteration schedule."""
     if mode == "newtonschulz" or x.shape[-2] != x.shape[-1]:
         y = newton_schulz5(x, rounding.noise16(philox.STREAM_NS_INPUT, tidx, x.shape))
+    elif mode == "thinky_polar_express":
+        y = polar_express(x, rounding.noise16(philox.STREAM_NS_INPUT, tidx, x.shape))
     elif mode == "legacy_newtonschulz":
         y = legacy_newton_schulz5(x, rounding.noise16(philox.STREAM_NS_INPUT, tidx, x.shape), rounding.noise16(philox.STREAM_NS_INPUT + 1, tidx, x.shape))
     else:

@@ -502,6 +502,23 @@ def make_legacy():
     torch.save(out, os.path.join(HERE, "ns5_bf16.pt"))
 
 
+def make_polar_express():
+    """zeroth_power_mode = "thinky_polar_express": square matrices take the ten-step schedule of msign (heavyball/utils.py:605-631,
+    :796-797), the others the default one; a trajectory under fp32 and one under bf16 gradients, and vectors from msign itself."""
+    shapes = [(16, 16), (16,), (24, 8), (8, 8)]
+    run_traj("muon_polar_express", heavyball.Muon, dict(weight_decay=0.01), shapes, torch.float32, 4, mode="thinky_polar_express")
+    run_traj("muon_polar_express_bf16grad_caution", heavyball.Muon, dict(caution=True), shapes, torch.bfloat16, 4, mode="thinky_polar_express")
+    out = {}
+    gen = torch.Generator().manual_seed(17)
+    for name, shape, dt in [("sq", (16, 16), torch.float32), ("sq64", (64, 64), torch.float32), ("sq96", (96, 96), torch.float32),
+                            ("sq64_bf16", (64, 64), torch.bfloat16), ("sq64_fp16", (64, 64), torch.float16)]:  # fmt: skip
+        G = (torch.randn(shape, generator=gen) * 1e-2).to(dt)
+        out[f"{name}/G"] = G.clone()
+        with half_rounding():
+            out[f"{name}/msign"] = heavyball.utils.msign(G.clone(), 10).clone()
+    torch.save(out, os.path.join(HERE, "msign.pt"))
+
+
 def make_muon():
     shapes = [(8, 16), (16,), (24, 8), (4, 3, 6)]
     run_traj("muon_default", heavyball.Muon, dict(weight_decay=0.01), shapes, torch.float32, 4)
@@ -589,7 +606,7 @@ def make_checkpoints():
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "soapnarrow", "muonfp16", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
+    which = sys.argv[1:] or ["layout", "scalars", "ecc", "traj", "variants", "palm", "clipcombo", "bothclips", "fp16unfused", "groupnorms", "muonnarrow", "soapmars", "soapsplit", "soapnarrow", "muonfp16", "polar", "switches", "ns5", "legacy", "muon", "soap", "ckpt"]
     if "layout" in which:
         make_layout()
     if "scalars" in which:
@@ -628,6 +645,8 @@ if __name__ == "__main__":
         make_legacy()
     if "muonfp16" in which:
         make_muon_fp16_gradients()
+    if "polar" in which:
+        make_polar_express()
     if "soap" in which:
         make_soap()
     if "ckpt" in which:

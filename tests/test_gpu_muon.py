@@ -250,6 +250,56 @@ def test_ns5_on_fp16_inputs_matches_reference_vectors(name):
         assert torch.equal(got, got.half().float()) and rel_fro(got, d[f"{name}/legacy"].float()) < NS_TOL
 
 
+def run_ns_steps(Gs, coeffs, rng_mode=_lib.RNG_HALF, seed=0, step=0, bases=None):
+    """hb_ns_batched_steps on the matrices ``Gs`` (fp32, bf16 or fp16 tensors) under one schedule of len(coeffs) iterations."""
+    L = _lib.lib()
+    n, n_steps = len(Gs), len(coeffs)
+    rows = (ctypes.c_int64 * n)(*[g.shape[0] for g in Gs])
+    cols = (ctypes.c_int64 * n)(*[g.shape[1] for g in Gs])
+    nbytes = ctypes.c_int64()
+    _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows, cols, ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
+    gs = [g.to(DEV, torch.float32).contiguous() for g in Gs]
+    outs = [torch.empty_like(g) for g in gs]
+    arr = (ctypes.c_float * (3 * n_steps * n))(*(ns_coeff_array(coeffs) * n))
+    flags = (ctypes.c_int32 * n)(*[{torch.bfloat16: _lib.NS_BF16_UPDATE, torch.float16: _lib.NS_F16_UPDATE}.get(g.dtype, 0) for g in Gs])
+    gp = (ctypes.c_void_p * n)(*[g.data_ptr() for g in gs])
+    op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    scale = (ctypes.c_float * n)(*[1.0] * n)
+    base = (ctypes.c_int64 * n)(*(bases or [0] * n))
+    _lib.check(L.hb_ns_batched_steps(n, gp, op, rows, cols, n_steps, arr, flags, 1e-7, scale, rng_mode, seed, step, base, ws.data_ptr(), nbytes.value, None),
+               "hb_ns_batched_steps")  # fmt: skip
+    torch.cuda.synchronize()
+    return [o.cpu() for o in outs]
+
+
+def test_polar_express_matches_reference_vectors_and_oracle():
+    """hb_ns_batched_steps under msign's ten-step schedule: against the vectors the reference computed (fp32, bf16 and float16
+    inputs, one call for all five), against the oracle on larger matrices of both tile classes, and with five steps of the default
+    schedule bit for bit what hb_ns5_batched gives."""
+    d = torch.load(os.path.join(GOLDEN, "msign.pt"), weights_only=True)
+    names = ["sq", "sq64", "sq96", "sq64_bf16", "sq64_fp16"]
+    outs = run_ns_steps([d[f"{k}/G"] for k in names], muon.POLAR_COEFFS)
+    for k, got in zip(names, outs):
+        print("case", k, flush=True)
+        assert rel_fro(got, d[f"{k}/msign"].float()) < NS_TOL
+    gen = torch.Generator().manual_seed(23)
+    Gs = [torch.randn(s, generator=gen) * 1e-2 for s in [(320, 320), (1100, 1100), (130, 515)]]
+    bases = [0, 4096 * 40, 4096 * 400]
+    outs = run_ns_steps(Gs, muon.POLAR_COEFFS, rng_mode=_lib.RNG_PHILOX, seed=5, step=3, bases=bases)
+    for k, (G, got) in enumerate(zip(Gs, outs)):
+        print("case", tuple(G.shape), flush=True)
+        r = PhiloxRounding(5, step=3, base=[bases[k]])
+        want = muon.polar_express(G.clone(), r.noise16(6, 0, G.shape))
+        assert rel_fro(got, want) < NS_TOL
+        sv = torch.linalg.svdvals(got.double())
+        assert sv.max() < 1.2 and sv.median() > 0.9  # ten steps bring the bulk of the spectrum to 1
+    five = run_ns_steps(Gs, muon.NS_COEFFS, rng_mode=_lib.RNG_PHILOX, seed=5, step=3, bases=bases)
+    for G, got, b in zip(Gs, five, bases):
+        alone = run_ns5(G, rng_mode=_lib.RNG_PHILOX, seed=5, step=3, base=b, scale=1.0)
+        assert torch.equal(got.view(torch.int32), alone.view(torch.int32))
+
+
 @pytest.mark.parametrize("legacy", [False, True])
 def test_ns5_fp16_input_and_output_roundings_are_the_oracles(legacy):
     """The float16 route through an identity schedule (a = 1, b = c = 0 makes an iteration return X): what comes back is the
@@ -462,8 +512,8 @@ def _random_muon_case(seed):
     rnd.shuffle(shapes)
     rounding = rnd.choice(["half", "philox"])
     mode = "newtonschulz"
-    if rnd.random() < 0.35:  # the legacy schedule, which square matrices take (heavyball/utils.py:790-795)
-        mode = "legacy_newtonschulz"
+    if rnd.random() < 0.35:  # the legacy schedule or msign's, which square matrices take (heavyball/utils.py:790-797)
+        mode = rnd.choice(["legacy_newtonschulz", "legacy_newtonschulz", "thinky_polar_express"])
         shapes += [(rnd.choice([8, 64, 130, 256]),) * 2, (3, 6, 18)]
     return kwargs, gdt, shapes, rounding, mode
 
