@@ -21,7 +21,7 @@ RNG_HALF, RNG_PHILOX = 0, 1
 STREAM_MARS_SR, STREAM_PARAM, STREAM_EXP_AVG, STREAM_EXP_AVG_SQ, STREAM_OLD_GRAD, STREAM_INIT_PARAM, STREAM_NS_INPUT = range(7)
 STREAM_CLIP, STREAM_EXP_AVG_SLOW, STREAM_UPDATE, STREAM_SOAP_ROTATE, STREAM_UPDATE_CLIP = 8, 9, 10, 11, 12
 STREAM_SOAP_GG, STREAM_SOAP_Q = 16, 17  # + 2 * side
-NS_LEGACY, NS_BF16_UPDATE, NS_F16_UPDATE = 1, 2, 4
+NS_LEGACY, NS_BF16_UPDATE, NS_F16_UPDATE, NS_APPLY_TO_PARAM, NS_CAUTIOUS_WD = 1, 2, 4, 8, 16
 NOALLOC_MAX_TENSORS = 8192  # HB_NOALLOC_MAX_TENSORS
 CAUTION_SLOTS = 32  # HB_CAUTION_SLOTS: counters per tensor in HbStepDesc.caution_count
 GEMM_ACCUMULATE, GEMM_SYMMETRIC = 1, 2
@@ -98,8 +98,8 @@ _PROTOTYPES = {
                                             POINTER(c_int32), c_float, POINTER(c_float), c_int32, c_uint64, c_uint32, POINTER(c_int64), c_void_p,
                                             c_int64, c_void_p]),
     "hb_ns_batched_steps": (ctypes.c_int, [c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64), c_int32, POINTER(c_float),
-                                           POINTER(c_int32), c_float, POINTER(c_float), c_int32, c_uint64, c_uint32, POINTER(c_int64), c_void_p,
-                                           c_int64, c_void_p]),
+                                           POINTER(c_int32), c_float, POINTER(c_float), POINTER(c_float), c_int32, c_uint64, c_uint32,
+                                           POINTER(c_int64), c_void_p, c_int64, c_void_p]),
     "hb_ns_product": (ctypes.c_int, [c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_void_p,
                                      c_int64, c_void_p]),
     "hb_ns5": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_int64, POINTER(c_float), c_int32, c_float, c_float, c_int32, c_uint64, c_uint32,

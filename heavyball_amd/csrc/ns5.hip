@@ -51,9 +51,13 @@ struct Problem {
   int tiles_m, tiles_n;              // tile grid of C
   int pos_begin;                     // where this run starts in the tile list of its XCD
   int t0, n_run;                     // the run: tiles t0 .. t0 + n_run - 1 of the matrix' tile list
-  int round_out;  // ModeFinal: the reference's update buffer is 16 bits wide (1 bf16, 2 fp16): cast and scaling round to it (to nearest)
+  // ModeFinal.  Bits 0-1: the reference's update buffer is 16 bits wide (1 bf16, 2 fp16): cast and scaling round to it (to nearest).
+  // kApplyToParam: F is the parameter and takes the step instead of receiving the update (mul_c, diag: its two factors).
+  int round_out;
 };
 static_assert(sizeof(Problem) % 16 == 0, "tables of problems are moved in 16-byte pieces");
+enum : int { kApplyToParam = 4, kCautiousWd = 8 };  // bits of Problem::round_out beside the update format
+
 // A table: this header, then the entries of XCD 0, of XCD 1, ...; entries [first[x], first[x + 1]) are XCD x's, in list order
 struct TableHeader {
   int first[9];
@@ -248,6 +252,36 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
         }
         prim[q] = h;
       }
+      // kApplyToParam: F is the fp32 parameter and takes p <- p * (1 - decay * lr) + update * (-lr), the tail of the reference's
+      // chain (heavyball/utils.py:2373-2390; the two factors travel in mul_c and diag, which this mode has no other use for), with
+      // the decay factor 1 where update and parameter disagree in sign under kCautiousWd.  The sub-tile's 16 parameter values
+      // are read before any of them is written, so that the loads are in flight together.
+      const bool apply = MODE == kModeFinal && (g.round_out & kApplyToParam) != 0;
+      float pv[16];
+      if (MODE == kModeFinal && apply) {
+#pragma unroll
+        for (int rb4 = 0; rb4 < 4; ++rb4) {
+          const int row = row_tile + rb4 * 8 + erow;
+          if (g.f_transposed) {
+            const float* src = g.F + (size_t)col * g.ldf + row;
+            if (col < g.f_rows && row + 3 < g.f_cols && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+              const float4 p4 = *reinterpret_cast<const float4*>(src);
+              pv[rb4 * 4 + 0] = p4.x; pv[rb4 * 4 + 1] = p4.y; pv[rb4 * 4 + 2] = p4.z; pv[rb4 * 4 + 3] = p4.w;
+            } else {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) pv[rb4 * 4 + r] = col < g.f_rows && row + r < g.f_cols ? src[r] : 0.0f;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pv[rb4 * 4 + r] = row + r < g.f_rows && col < g.f_cols ? g.F[(size_t)(row + r) * g.ldf + col] : 0.0f;
+          }
+        }
+      }
+      auto stepped = [&](float p, float u) {
+        float om = g.mul_c;
+        if ((g.round_out & kCautiousWd) && ((f2u(p) ^ f2u(u)) >> 31)) om = 1.0f;
+        return p * om + u * g.diag;
+      };
 #pragma unroll
       for (int rb4 = 0; rb4 < 4; ++rb4) {
         const int row = row_tile + rb4 * 8 + erow;
@@ -259,10 +293,14 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
               o[r] = acc[i][j][rb4 * 4 + r];  // one K chunk of a split product: summed and rounded by ns_split_reduce_kernel
             } else {
               o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
-              if (g.round_out == 1) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
-              else if (g.round_out == 2)  // fp16: the cast leaves bf16's range (subnormals, overflow), then the product rounds again
-                o[r] = f16_to_f32(f32_to_f16_rne(f16_to_f32(f32_to_f16_rne(bf16_to_f32(prim[rb4 * 4 + r]))) * g.scale));
+              if ((g.round_out & 3) == 1) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
+              else if ((g.round_out & 3) == 2)  // fp16: the cast leaves bf16's range (subnormals, overflow), then the product rounds again
+                o[r] = f16_to_f32(f32_to_f16_rne(f16_to_f32(f32_to_f16_rne_plain(bf16_to_f32(prim[rb4 * 4 + r]))) * g.scale));
             }
+          }
+          if (MODE == kModeFinal && apply) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = stepped(pv[rb4 * 4 + r], o[r]);
           }
           if (g.f_transposed) {
             // the 4 consecutive rows of X are 16 contiguous bytes of the output's row `col`
@@ -1052,8 +1090,8 @@ static size_t table_bytes(const std::vector<NsPlan>& plans) {
 // coeffs_host: 3 * n_steps floats per matrix when per_matrix, else one table of that many; flags likewise
 static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols, int n_steps,
                             const float* coeffs_host, const int32_t* flags, bool per_matrix, float eps, const float* post_scale,
-                            int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
-                            int64_t workspace_bytes, hipStream_t s, const char* who) {
+                            const float* param_step, int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base,
+                            void* workspace, int64_t workspace_bytes, hipStream_t s, const char* who) {
   if (n_mats <= 0 || !g || !out || !rows || !cols || !coeffs_host || !flags || !post_scale || !flat_base || !workspace)
     return set_error(HB_EINVAL, "%s: null pointer or empty batch", who);
   if (rng_mode != HB_RNG_HALF && rng_mode != HB_RNG_PHILOX) return set_error(HB_EINVAL, "%s: bad rng_mode", who);
@@ -1061,9 +1099,15 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return set_error(HB_EINVAL, "%s: workspace must be 256-byte aligned", who);
   auto flag_of = [&](int i) { return flags[per_matrix ? i : 0]; };
   auto coeff_of = [&](int i, int k) { return coeffs_host[(per_matrix ? (size_t)i * 3 * n_steps : 0) + k]; };
-  for (int i = 0; i < n_mats; ++i)
-    if ((flag_of(i) & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) || (flag_of(i) & (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) == (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE))
+  for (int i = 0; i < n_mats; ++i) {
+    const int f = flag_of(i);
+    if ((f & ~(HB_NS_LEGACY | HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE | HB_NS_APPLY_TO_PARAM | HB_NS_CAUTIOUS_WD)) ||
+        (f & (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE)) == (HB_NS_BF16_UPDATE | HB_NS_F16_UPDATE))
       return set_error(HB_EINVAL, "%s: unknown flag bits, or both update formats at once", who);
+    if ((f & HB_NS_APPLY_TO_PARAM) && (!param_step || g[i] == out[i]))
+      return set_error(HB_EINVAL, "%s: HB_NS_APPLY_TO_PARAM needs param_step and an output that is not the input", who);
+    if ((f & HB_NS_CAUTIOUS_WD) && !(f & HB_NS_APPLY_TO_PARAM)) return set_error(HB_EINVAL, "%s: HB_NS_CAUTIOUS_WD goes with HB_NS_APPLY_TO_PARAM", who);
+  }
   for (int i = 0; i < n_mats; ++i) {
     if (!g[i] || !out[i]) return set_error(HB_EINVAL, "%s: null matrix pointer at %d", who, i);
     if (rows[i] <= 0 || cols[i] <= 0 || rows[i] > (1 << 20) || cols[i] > (1 << 20)) return set_error(HB_EINVAL, "%s: bad shape at %d", who, i);
@@ -1217,6 +1261,11 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
             q.F = out[i]; q.f_transposed = p.rows > p.cols; q.ldf = (int)p.cols; q.f_rows = (int)p.rows; q.f_cols = (int)p.cols;
             q.scale = post_scale[i];
             q.round_out = (flag_of(i) & HB_NS_BF16_UPDATE) ? 1 : (flag_of(i) & HB_NS_F16_UPDATE) ? 2 : 0;
+            if (flag_of(i) & HB_NS_APPLY_TO_PARAM) {
+              q.round_out |= kApplyToParam | ((flag_of(i) & HB_NS_CAUTIOUS_WD) ? kCautiousWd : 0);
+              q.mul_c = param_step[0];
+              q.diag = param_step[1];
+            }
           }
           probs[k] = q;
         }
@@ -1281,7 +1330,7 @@ extern "C" int hb_ns5_batched(int32_t n_mats, const float* const* g, float* cons
                               const float* coeffs_host, int32_t legacy, float eps, const float* post_scale, int32_t rng_mode,
                               uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                               void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, &legacy, false, eps, post_scale, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, &legacy, false, eps, post_scale, nullptr, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched");
 }
 
@@ -1289,21 +1338,21 @@ extern "C" int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float
                                     const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
                                     uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                                     void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, flags, true, eps, post_scale, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, flags, true, eps, post_scale, nullptr, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched_mixed");
 }
 
 extern "C" int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                                    int32_t n_steps, const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale,
-                                   int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
-                                   int64_t workspace_bytes, void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, n_steps, coeffs_host, flags, true, eps, post_scale, rng_mode, seed, step, flat_base,
-                              workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns_batched_steps");
+                                   const float* param_step, int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base,
+                                   void* workspace, int64_t workspace_bytes, void* stream_) {
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, n_steps, coeffs_host, flags, true, eps, post_scale, param_step, rng_mode, seed, step,
+                              flat_base, workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns_batched_steps");
 }
 
 extern "C" int hb_ns5(const float* g, float* out, int64_t rows, int64_t cols, const float* coeffs_host, int32_t legacy, float eps,
                       float post_scale, int32_t rng_mode, uint64_t seed, uint32_t step, int64_t flat_base, void* workspace,
                       int64_t workspace_bytes, void* stream_) {
-  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, 5, coeffs_host, &legacy, false, eps, &post_scale, rng_mode, seed, step, &flat_base, workspace,
+  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, 5, coeffs_host, &legacy, false, eps, &post_scale, nullptr, rng_mode, seed, step, &flat_base, workspace,
                               workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5");
 }

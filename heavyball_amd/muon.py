@@ -97,6 +97,9 @@ class Muon(HBOptimizer):
 
     #: upper bound on the Newton-Schulz scratch of one grouped call; a bucket whose matrices need more is split
     ns_workspace_limit = 16 << 30
+    #: let the last Newton-Schulz product apply the step to fp32 parameters itself where the chain allows it (same arithmetic as
+    #: hb_update_param; False keeps the two launches apart, which tests use to compare the two routes)
+    fuse_update_into_newton_schulz = True
 
     def _ns_parts(self, L, mats):
         """Splits ``[(index, rows, cols), ...]`` into runs whose scratch stays under ``ns_workspace_limit``."""
@@ -203,6 +206,7 @@ class Muon(HBOptimizer):
             for (b, _, gdt), res in zip(work, (yield from self._clip_gradients_gen(L, group, work, step, gathered=mars))):
                 clipped[(id(b), gdt)] = res
         keep = []
+        stepped = set()  # (bucket, tensor) whose parameter the last Newton-Schulz product has already updated
         tables = {}  # (bucket, gradient dtype) -> device table of gradient pointers
         for b, items, by_dtype in prepared:
             offsets, numel = b.slab.meta()
@@ -235,6 +239,13 @@ class Muon(HBOptimizer):
                 # with 16-bit gradients the reference's update buffer has their dtype and Newton-Schulz normalises it there
                 # (per matrix: a bucket may hold gradients of several dtypes)
                 ns_flags = {i: _NS_UPDATE_FLAG[gdt] for gdt, lst in by_dtype.items() for i, _ in lst}
+                # an fp32 parameter that nothing else looks at between Newton-Schulz and update_param_ (no caution, whose mask needs
+                # the finished update of the whole tensor, and no clip of the update) takes its step in the epilogue of the last
+                # product: the update is never written out and read back
+                fuse_tail = (self.fuse_update_into_newton_schulz and not group["caution"] and self.update_clipping is None and not pecc
+                             and b.param_dtype == torch.float32)  # fmt: skip
+                tail_flags = (_lib.NS_APPLY_TO_PARAM | (_lib.NS_CAUTIOUS_WD if flags & _lib.FLAG_CAUTIOUS_WD else 0)) if fuse_tail else 0
+                param_step = (ctypes.c_float * 2)(omdl, neg_lr)
                 mats = []
                 for i, p, _ in items:
                     if p.dim() < 2:
@@ -250,16 +261,19 @@ class Muon(HBOptimizer):
                     rows_a = (ctypes.c_int64 * n)(*[r for _, r, _ in part])
                     cols_a = (ctypes.c_int64 * n)(*[c for _, _, c in part])
                     ptrs = (ctypes.c_void_p * n)(*[b.slab.view("_update", i).data_ptr() for i, _, _ in part])
+                    outs = (ctypes.c_void_p * n)(*[b.slab.view("param", i).data_ptr() for i, _, _ in part]) if fuse_tail else ptrs
                     scale = (ctypes.c_float * n)(*[max(1, r / c) ** 0.5 for _, r, c in part])  # heavyball/utils.py:808-809
                     base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
                     arr = (ctypes.c_float * (3 * n_steps * n))(*[x for lg in legacy for x in coeff_tables["polar" if n_steps == 10 else lg]])
-                    flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) for (i, _, _), lg in zip(part, legacy)])
+                    flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) | tail_flags for (i, _, _), lg in zip(part, legacy)])
                     nbytes = ctypes.c_int64()
                     _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows_a, cols_a, ctypes.byref(nbytes)))
                     ws = self._ws(b.device, nbytes.value)
-                    _lib.check(L.hb_ns_batched_steps(n, ptrs, ptrs, rows_a, cols_a, n_steps, arr, flag_a, 1e-7, scale, self._rng_mode(),
-                                                     self.rng_seed, int(step) & 0xFFFFFFFF, base, ws.data_ptr(), ws.numel(), stream),
-                               "hb_ns_batched_steps")  # fmt: skip
+                    _lib.check(L.hb_ns_batched_steps(n, ptrs, outs, rows_a, cols_a, n_steps, arr, flag_a, 1e-7, scale, param_step,
+                                                     self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF, base, ws.data_ptr(),
+                                                     ws.numel(), stream), "hb_ns_batched_steps")  # fmt: skip
+                if fuse_tail:
+                    stepped.update((id(b), i) for i, _, _ in mats)
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group
             keep.append((yield (self.update_clipping, "_update", [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared])))
             for b, items, by_dtype in prepared:
@@ -280,7 +294,9 @@ class Muon(HBOptimizer):
             with torch.cuda.device(b.device):
                 # p <- p * (1 - decay * lr) + update * (-lr) for everything (heavyball/utils.py:2373-2406)
                 for gdt, lst in by_dtype.items():
-                    act = tuple(i for i, _ in lst)
+                    act = tuple(i for i, _ in lst if (id(b), i) not in stepped)  # the others took their step inside Newton-Schulz
+                    if not act:
+                        continue
                     chunks, n_chunks = b.slab.chunks(act)
                     table = tables[(id(b), gdt)]
                     d = _lib.HbStepDesc()

@@ -256,7 +256,7 @@ int hb_momentum(void* momentum, void* momentum_corr, int32_t momentum_fmt, float
  * cast to fp16 and scaled there (two roundings to nearest).  With HB_NS_LEGACY only the norm is an fp16 value (its division
  * runs in fp32).  The two update flags exclude each other.
  */
-enum { HB_NS_LEGACY = 1, HB_NS_BF16_UPDATE = 2, HB_NS_F16_UPDATE = 4 };
+enum { HB_NS_LEGACY = 1, HB_NS_BF16_UPDATE = 2, HB_NS_F16_UPDATE = 4, HB_NS_APPLY_TO_PARAM = 8, HB_NS_CAUTIOUS_WD = 16 };
 int hb_ns5_workspace_bytes(int64_t rows, int64_t cols, int64_t* bytes);
 int hb_ns5(const float* g, float* out, int64_t rows, int64_t cols, const float* coeffs_host, int32_t legacy, float eps,
            float post_scale, int32_t rng_mode, uint64_t seed, uint32_t step, int64_t flat_base, void* workspace,
@@ -289,11 +289,16 @@ int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* ou
  * replaces msign (heavyball/utils.py:605-631), the ten-step "Polar Express" schedule that square matrices take under
  * zeroth_power_mode = "thinky_polar_express" (:796-797), followed by the same post-scale; normalisation, input rounding and
  * the iteration are those of hb_ns5.  Same workspace as hb_ns5_batched for the same shapes; hb_ns5_batched_mixed is this call
- * with n_steps = 5. */
+ * with n_steps = 5 and param_step = NULL.
+ * HB_NS_APPLY_TO_PARAM in a matrix' flag word fuses the chain's tail into the last product: out[i] is then the matrix' fp32
+ * PARAMETER (not g[i]) and takes p <- p * param_step[0] + update * param_step[1], i.e. update_param_ without caution
+ * (heavyball/utils.py:2373-2406) with param_step = {1 - decay * lr, -lr} in HOST memory, in the arithmetic of hb_update_param;
+ * the update itself is not written anywhere.  HB_NS_CAUTIOUS_WD with it: the first factor is 1 where update and parameter
+ * differ in sign (cautious weight decay). */
 int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                         int32_t n_steps, const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale,
-                        int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace,
-                        int64_t workspace_bytes, void* stream);
+                        const float* param_step, int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base,
+                        void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Test hook: ONE product of the Newton-Schulz iteration on bf16 operands (row-major, K contiguous: A [M, K], B [N, K]) through
  * the kernel of the given tile class (128 or 256), so that a test can put the same product through both kernels, whose

@@ -267,7 +267,7 @@ def run_ns_steps(Gs, coeffs, rng_mode=_lib.RNG_HALF, seed=0, step=0, bases=None)
     op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
     scale = (ctypes.c_float * n)(*[1.0] * n)
     base = (ctypes.c_int64 * n)(*(bases or [0] * n))
-    _lib.check(L.hb_ns_batched_steps(n, gp, op, rows, cols, n_steps, arr, flags, 1e-7, scale, rng_mode, seed, step, base, ws.data_ptr(), nbytes.value, None),
+    _lib.check(L.hb_ns_batched_steps(n, gp, op, rows, cols, n_steps, arr, flags, 1e-7, scale, None, rng_mode, seed, step, base, ws.data_ptr(), nbytes.value, None),
                "hb_ns_batched_steps")  # fmt: skip
     torch.cuda.synchronize()
     return [o.cpu() for o in outs]
@@ -486,6 +486,39 @@ def test_muon_optimizer_matches_oracle(variant, rounding):
                 # decay moves both sides identically up to the parameter drift; compare the steps
                 assert rel_fro(got, want) < NS_TOL, (k, i, rel_fro(got, want))
         assert opt.param_groups[0]["step"] is None
+
+
+@pytest.mark.parametrize("kwargs,gdt", [(dict(lr=0.02, weight_decay=0.1), torch.float32),
+                                        (dict(lr=0.02, weight_decay=0.1, cautious_weight_decay=True, mars=True), torch.bfloat16),
+                                        (dict(lr=0.02, ecc="bf16+8", nesterov=False), torch.float16)])
+def test_step_inside_the_last_product_equals_the_separate_update(kwargs, gdt):
+    """Where the chain allows it the last Newton-Schulz product applies p <- p (1 - decay lr) - lr u itself
+    (HB_NS_APPLY_TO_PARAM) instead of writing u for hb_update_param to read back: the same arithmetic on the same values, so
+    the parameters agree bit for bit with the two-launch route, over wide, tall, ragged and stacked matrices of both tile
+    classes, with vectors (which keep the separate update) in the same bucket."""
+    import heavyball_amd
+    from tests import helpers as H
+
+    shapes = [(192, 320), (64,), (320, 128), (8, 6, 24), (130, 70), (1100, 1024), (1, 5), (7,)]
+    print("case", kwargs, gdt, flush=True)
+    host, pa = H.make_params(shapes, DEV)
+    _, pb = H.make_params(shapes, DEV)
+    oa, ob = heavyball_amd.Muon(pa, **kwargs), heavyball_amd.Muon(pb, **kwargs)
+    ob.fuse_update_into_newton_schulz = False
+    for o in (oa, ob):
+        o.rounding, o.rng_seed = "philox", 77
+    for p in pa + pb:
+        p.grad_dtype = None
+    for k in range(1, 4):
+        grads = H.make_grads(shapes, k, gdt, 1e-2)
+        for p, q, g in zip(pa, pb, grads):
+            p.grad, q.grad = g.to(DEV), g.to(DEV).clone()
+        oa.step()
+        ob.step()
+        torch.cuda.synchronize()
+        for i, (p, q) in enumerate(zip(pa, pb)):
+            assert torch.equal(p.detach().view(torch.int32), q.detach().view(torch.int32)), (k, i, shapes[i])
+    assert all(not torch.equal(p.detach().cpu(), h) for p, h in zip(pa, host))  # and they did move
 
 
 def _random_muon_case(seed):
