@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("HBSTEP_LIB") or os.path.join(_HERE, "libhbstep.so")
 
 # include/hbstep.h
-ABI_VERSION = 10  # HB_ABI_VERSION this binding was written against
+ABI_VERSION = 11  # HB_ABI_VERSION this binding was written against
 FMT_F32, FMT_BF16, FMT_F16, FMT_ECC_BF16_8, FMT_ECC_BF16_16, FMT_ECC_F16_8, FMT_ECC_F16_16 = range(7)
 ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD, FLAG_MARS_ONLY = 1, 2, 4, 8, 16, 32, 64, 128
@@ -89,6 +89,9 @@ _PROTOTYPES = {
     "hb_nesterov_ema": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_void_p]),
     "hb_momentum": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
                                    c_int32, c_float, c_float, c_int32, c_uint64, c_uint32, c_void_p]),
+    "hb_momentum_sumsq": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+                                         c_int32, c_float, c_float, c_int32, c_uint64, c_uint32, c_void_p, c_void_p]),
+    "hb_momentum_sumsq_parts_per_chunk": (ctypes.c_int, []),
     "hb_ns5_workspace_bytes": (ctypes.c_int, [c_int64, c_int64, POINTER(c_int64)]),
     "hb_ns5_batched_workspace_bytes": (ctypes.c_int, [c_int32, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
     "hb_ns5_batched": (ctypes.c_int, [c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64), POINTER(c_float),
@@ -98,8 +101,8 @@ _PROTOTYPES = {
                                             POINTER(c_int32), c_float, POINTER(c_float), c_int32, c_uint64, c_uint32, POINTER(c_int64), c_void_p,
                                             c_int64, c_void_p]),
     "hb_ns_batched_steps": (ctypes.c_int, [c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64), c_int32, POINTER(c_float),
-                                           POINTER(c_int32), c_float, POINTER(c_float), POINTER(c_float), c_int32, c_uint64, c_uint32,
-                                           POINTER(c_int64), c_void_p, c_int64, c_void_p]),
+                                           POINTER(c_int32), c_float, POINTER(c_float), POINTER(c_float), POINTER(c_void_p), POINTER(c_int32),
+                                           c_int32, c_uint64, c_uint32, POINTER(c_int64), c_void_p, c_int64, c_void_p]),
     "hb_ns_product": (ctypes.c_int, [c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_void_p,
                                      c_int64, c_void_p]),
     "hb_ns5": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_int64, POINTER(c_float), c_int32, c_float, c_float, c_int32, c_uint64, c_uint32,

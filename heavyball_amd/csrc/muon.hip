@@ -27,68 +27,95 @@ __global__ __launch_bounds__(kMThreads) void momentum_kernel(char* __restrict__ 
                                                               const char* __restrict__ grad, const char* const* __restrict__ grad_ptrs, int gf,
                                                               const int64_t* __restrict__ offsets, const int64_t* __restrict__ numel,
                                                               const int2* __restrict__ chunks, int64_t n_chunks, float a, float oma, int mode,
-                                                              Rng rng) {
+                                                              Rng rng, double* __restrict__ sumsq_parts) {
   for (int64_t w = blockIdx.x; w < n_chunks * kMSub; w += gridDim.x) {
     const int2 ent = chunks[w / kMSub];
     const int64_t local0 = (int64_t)ent.y * HB_CHUNK + (int64_t)(w % kMSub) * kMWork;
     const int64_t rem = numel[ent.x] - local0;
-    if (rem <= 0) continue;  // a work unit behind the end of the tensor's last chunk
+    // sumsq_parts: the sum of squares of the update this wavefront writes, one double per wavefront and work unit (no barrier,
+    // no atomics: whoever adds them up gets the same sum in every run); zero for a unit or a wavefront past the tensor's end
+    double* const part = sumsq_parts ? sumsq_parts + w * (kMThreads / 64) + (threadIdx.x >> 6) : nullptr;
+    if (rem <= 0) {  // a work unit behind the end of the tensor's last chunk
+      if (part && (threadIdx.x & 63) == 0) *part = 0.0;
+      continue;
+    }
     const int valid = rem < kMWork ? (int)rem : kMWork;
     const int64_t flat0 = offsets[ent.x] + local0;
     const bool g_slab = grad_ptrs == nullptr;
     const char* gbase = g_slab ? grad : grad_ptrs[ent.x];
     const int64_t g0 = g_slab ? flat0 : local0;
     const int e = threadIdx.x * kME;
-    if (e >= valid) continue;
-    const int64_t idx = flat0 + e;
-    RawT<kME> rm;
-    float m[kME], g[kME], u[kME];
-    raw_load<MF>(rm, mf, mom, mom_corr, idx);
-    if (g_slab || e + kME <= valid) {  // a whole run: one wide load (gradient buffers are 16-byte aligned)
-      RawT<kME> rg;
-      raw_load<kDyn>(rg, gf, gbase, nullptr, g0 + e);
-      raw_decode<kDyn>(rg, gf, g);
-    } else {  // last, partial run of a gradient that is not padded
+    double ss = 0.0;  // this lane's share of the unit's sum of squares; lanes past the tensor's end add nothing
+    if (e < valid) {
+      const int64_t idx = flat0 + e;
+      RawT<kME> rm;
+      float m[kME], g[kME], u[kME];
+      raw_load<MF>(rm, mf, mom, mom_corr, idx);
+      if (g_slab || e + kME <= valid) {  // a whole run: one wide load (gradient buffers are 16-byte aligned)
+        RawT<kME> rg;
+        raw_load<kDyn>(rg, gf, gbase, nullptr, g0 + e);
+        raw_decode<kDyn>(rg, gf, g);
+      } else {  // last, partial run of a gradient that is not padded
 #pragma unroll
-      for (int j = 0; j < kME; ++j) g[j] = e + j < valid ? load_elem(gbase, gf, g0 + e + j) : 0.0f;
-    }
-    raw_decode<MF>(rm, mf, m);
+        for (int j = 0; j < kME; ++j) g[j] = e + j < valid ? load_elem(gbase, gf, g0 + e + j) : 0.0f;
+      }
+      raw_decode<MF>(rm, mf, m);
 #pragma unroll
-    for (int j = 0; j < kME; ++j) {
-      if (mode == HB_MOM_NESTEROV_EMA) {
-        m[j] = m[j] * oma + g[j] * a;  // heavyball/utils.py:1048 via _lerp (:1847)
-        u[j] = g[j] + m[j] * 1.0f;     // stochastic_add_(grad, ema32, 1), heavyball/utils.py:1127-1130
-      } else if (mode == HB_MOM_EMA) {
-        m[j] = m[j] * oma + g[j] * a;
-        u[j] = m[j];
-      } else {  // a carries beta
-        m[j] = m[j] * a + g[j];
-        u[j] = mode == HB_MOM_HEAVYBALL ? m[j] : g[j] + m[j] * a;
+      for (int j = 0; j < kME; ++j) {
+        if (mode == HB_MOM_NESTEROV_EMA) {
+          m[j] = m[j] * oma + g[j] * a;  // heavyball/utils.py:1048 via _lerp (:1847)
+          u[j] = g[j] + m[j] * 1.0f;     // stochastic_add_(grad, ema32, 1), heavyball/utils.py:1127-1130
+        } else if (mode == HB_MOM_EMA) {
+          m[j] = m[j] * oma + g[j] * a;
+          u[j] = m[j];
+        } else {  // a carries beta
+          m[j] = m[j] * a + g[j];
+          u[j] = mode == HB_MOM_HEAVYBALL ? m[j] : g[j] + m[j] * a;
+        }
+      }
+      // the update buffer of the reference has the gradient's dtype: a 16-bit gradient rounds the update as
+      // copy_stochastic_ does (bf16: stochastic, fp16: to nearest), heavyball/utils.py:2363-2370
+      if (gf == HB_FMT_BF16) {
+        const Noise<kME> rn = rng.noise<kME>(idx, HB_STREAM_MARS_SR);
+#pragma unroll
+        for (int j = 0; j < kME; ++j) u[j] = bf16_to_f32(sr_bf16(u[j], rn.bits16(j)));
+      } else if (gf == HB_FMT_F16) {
+#pragma unroll
+        for (int j = 0; j < kME; ++j) u[j] = f16_to_f32(f32_to_f16_rne(u[j]));
+      }
+      const bool state_rounds = MF == kDyn;  // bf16 storage rounds stochastically, ECC pairs draw their correction
+      const Noise<kME> rn_m = state_rounds ? rng.noise<kME>(idx, HB_STREAM_EXP_AVG) : Noise<kME>{};
+      raw_put<MF>(mf, m, rn_m, mom, mom_corr, idx);
+      raw_put<HB_FMT_F32>(0, u, Noise<kME>{}, reinterpret_cast<char*>(upd), nullptr, idx);
+      if (part) {
+#pragma unroll
+        for (int j = 0; j < kME; ++j)
+          if (e + j < valid) ss += (double)u[j] * (double)u[j];
       }
     }
-    // the update buffer of the reference has the gradient's dtype: a 16-bit gradient rounds the update as
-    // copy_stochastic_ does (bf16: stochastic, fp16: to nearest), heavyball/utils.py:2363-2370
-    if (gf == HB_FMT_BF16) {
-      const Noise<kME> rn = rng.noise<kME>(idx, HB_STREAM_MARS_SR);
-#pragma unroll
-      for (int j = 0; j < kME; ++j) u[j] = bf16_to_f32(sr_bf16(u[j], rn.bits16(j)));
-    } else if (gf == HB_FMT_F16) {
-#pragma unroll
-      for (int j = 0; j < kME; ++j) u[j] = f16_to_f32(f32_to_f16_rne(u[j]));
+    if (part) {  // every lane of the wavefront is here: a wavefront-wide sum
+      ss = wave_sum(ss);
+      if ((threadIdx.x & 63) == 0) *part = ss;
     }
-    const bool state_rounds = MF == kDyn;  // bf16 storage rounds stochastically, ECC pairs draw their correction
-    const Noise<kME> rn_m = state_rounds ? rng.noise<kME>(idx, HB_STREAM_EXP_AVG) : Noise<kME>{};
-    raw_put<MF>(mf, m, rn_m, mom, mom_corr, idx);
-    raw_put<HB_FMT_F32>(0, u, Noise<kME>{}, reinterpret_cast<char*>(upd), nullptr, idx);
   }
 }
 
 }  // namespace hb
 
+extern "C" int hb_momentum_sumsq_parts_per_chunk(void) { return hb::kMSub * (hb::kMThreads / 64); }
+
 extern "C" int hb_momentum(void* momentum, void* momentum_corr, int32_t momentum_fmt, float* update, const void* grad,
                            const void* const* grad_ptrs, int32_t grad_fmt, const int64_t* offsets, const int64_t* numel, const int32_t* chunks,
                            int64_t n_chunks, int32_t mode, float a, float one_minus_a, int32_t rng_mode, uint64_t seed, uint32_t step,
                            void* stream_) {
+  return hb_momentum_sumsq(momentum, momentum_corr, momentum_fmt, update, grad, grad_ptrs, grad_fmt, offsets, numel, chunks, n_chunks, mode, a,
+                           one_minus_a, rng_mode, seed, step, nullptr, stream_);
+}
+
+extern "C" int hb_momentum_sumsq(void* momentum, void* momentum_corr, int32_t momentum_fmt, float* update, const void* grad,
+                                 const void* const* grad_ptrs, int32_t grad_fmt, const int64_t* offsets, const int64_t* numel,
+                                 const int32_t* chunks, int64_t n_chunks, int32_t mode, float a, float one_minus_a, int32_t rng_mode,
+                                 uint64_t seed, uint32_t step, double* sumsq_parts, void* stream_) {
   using namespace hb;
   if (mode < HB_MOM_NESTEROV_EMA || mode > HB_MOM_NESTEROV_HEAVYBALL) return set_error(HB_EINVAL, "hb_momentum: bad mode");
   if (n_chunks < 0) return set_error(HB_EINVAL, "hb_momentum: negative size");
@@ -110,9 +137,11 @@ extern "C" int hb_momentum(void* momentum, void* momentum_corr, int32_t momentum
   const char* const* gp = reinterpret_cast<const char* const*>(grad_ptrs);
   const int2* ch = reinterpret_cast<const int2*>(chunks);
   if (momentum_fmt == HB_FMT_F32)
-    momentum_kernel<HB_FMT_F32><<<grid, kMThreads, 0, s>>>(m, mc, momentum_fmt, update, g, gp, grad_fmt, offsets, numel, ch, n_chunks, a, one_minus_a, mode, rng);
+    momentum_kernel<HB_FMT_F32><<<grid, kMThreads, 0, s>>>(m, mc, momentum_fmt, update, g, gp, grad_fmt, offsets, numel, ch, n_chunks, a, one_minus_a, mode, rng,
+                                                           sumsq_parts);
   else
-    momentum_kernel<kDyn><<<grid, kMThreads, 0, s>>>(m, mc, momentum_fmt, update, g, gp, grad_fmt, offsets, numel, ch, n_chunks, a, one_minus_a, mode, rng);
+    momentum_kernel<kDyn><<<grid, kMThreads, 0, s>>>(m, mc, momentum_fmt, update, g, gp, grad_fmt, offsets, numel, ch, n_chunks, a, one_minus_a, mode, rng,
+                                                     sumsq_parts);
   return check_launch("hb_momentum");
 }
 

@@ -673,11 +673,12 @@ struct PrepItem {
   const float* g;     // the gradient [rows, cols]
   uint16_t* X;        // [m, n] padded, m <= n
   uint16_t* Xt;       // [n, m] padded
-  double* partial;    // n_blocks partial sums of squares
+  const double* partial;  // n_blocks partial sums of squares (the call's own scratch, or the caller's)
   float* norm;        // max(||g||_F, eps)
   int64_t flat_base;  // Philox flat index of g[0, 0]
   int rows, cols, ldx, ldxt, transpose;
-  int n_blocks, block_begin;  // sum of squares: this matrix owns workgroups [block_begin, block_begin + n_blocks)
+  int n_blocks, block_begin;  // sum of squares: n_blocks partial sums; this matrix owns workgroups [block_begin, block_begin + sum_blocks)
+  int sum_blocks;             // ... n_blocks of them, or none when the caller brought the partial sums
   int tiles_c, tile_begin;    // conversion: 64 x 64 tiles, tiles_c per tile row, first workgroup id
   int legacy;                 // two stochastic rounds (legacy_zeropower_via_newtonschulz5) instead of one
   // the reference's update buffer is 16 bits wide.  1 (bf16): norm and quotient are bf16 values (to nearest), no stochastic round.
@@ -701,8 +702,8 @@ __global__ __launch_bounds__(256) void ns_sumsq_kernel(const PrepGroup grp) {
   while (pi + 1 < n_items && (int)blockIdx.x >= ka->it[pi + 1].block_begin) ++pi;
   const float* __restrict__ g = ka->it[pi].g;
   const int64_t n = (int64_t)ka->it[pi].rows * ka->it[pi].cols;
-  const int nb = ka->it[pi].n_blocks, b = blockIdx.x - ka->it[pi].block_begin;
-  double* __restrict__ partial = ka->it[pi].partial;
+  const int nb = ka->it[pi].sum_blocks, b = blockIdx.x - ka->it[pi].block_begin;
+  double* __restrict__ partial = const_cast<double*>(ka->it[pi].partial);
   __shared__ double lds[4];
   double acc = 0.0;
   const int64_t n4 = (reinterpret_cast<uintptr_t>(g) & 15) == 0 ? n >> 2 : 0;  // 128-bit loads when the buffer allows
@@ -721,19 +722,31 @@ __global__ __launch_bounds__(256) void ns_sumsq_kernel(const PrepGroup grp) {
   if (threadIdx.x == 0) partial[b] = lds[0] + lds[1] + lds[2] + lds[3];
 }
 
-__global__ __launch_bounds__(256) void ns_norm_final_kernel(const PrepGroup grp) {
+// One workgroup per matrix adds the partial sums in a fixed order.  A caller's partial sums come a few per chunk of 4096
+// elements (150 thousand for an embedding of 38 M elements), so the workgroup is 1024 lanes wide and every lane keeps eight loads
+// in flight; a lane's terms and the order of the final additions depend on nothing but the count.
+constexpr int kNormThreads = 1024;
+__global__ __launch_bounds__(kNormThreads) void ns_norm_final_kernel(const PrepGroup grp) {
   const prep_ptr_t ka = (prep_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
   const int pi = blockIdx.x;
   const double* __restrict__ partial = ka->it[pi].partial;
   const int n = ka->it[pi].n_blocks;
-  __shared__ double lds[4];
+  __shared__ double lds[kNormThreads / 64];
   double acc = 0.0;
-  for (int i = threadIdx.x; i < n; i += 256) acc += partial[i];
+  for (int i0 = threadIdx.x; i0 < n; i0 += kNormThreads * 8) {
+    double v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = i0 + u * kNormThreads < n ? partial[i0 + u * kNormThreads] : 0.0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u];
+  }
   acc = wave_sum(acc);
   if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
   __syncthreads();
   if (threadIdx.x == 0) {
-    float nrm = __builtin_sqrtf((float)(lds[0] + lds[1] + lds[2] + lds[3]));
+    double total = 0.0;
+    for (int k = 0; k < kNormThreads / 64; ++k) total += lds[k];
+    float nrm = __builtin_sqrtf((float)total);
     float eps = grp.eps;
     // a 16-bit tensor's norm is a value of its dtype; so is the clamp bound, except under the legacy schedule, whose division
     // promotes both sides to fp32 first (heavyball/utils.py:1174-1179, :1190)
@@ -1090,8 +1103,9 @@ static size_t table_bytes(const std::vector<NsPlan>& plans) {
 // coeffs_host: 3 * n_steps floats per matrix when per_matrix, else one table of that many; flags likewise
 static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols, int n_steps,
                             const float* coeffs_host, const int32_t* flags, bool per_matrix, float eps, const float* post_scale,
-                            const float* param_step, int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base,
-                            void* workspace, int64_t workspace_bytes, hipStream_t s, const char* who) {
+                            const float* param_step, const double* const* sumsq_parts, const int32_t* n_sumsq_parts, int32_t rng_mode,
+                            uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
+                            hipStream_t s, const char* who) {
   if (n_mats <= 0 || !g || !out || !rows || !cols || !coeffs_host || !flags || !post_scale || !flat_base || !workspace)
     return set_error(HB_EINVAL, "%s: null pointer or empty batch", who);
   if (rng_mode != HB_RNG_HALF && rng_mode != HB_RNG_PHILOX) return set_error(HB_EINVAL, "%s: bad rng_mode", who);
@@ -1108,7 +1122,9 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
       return set_error(HB_EINVAL, "%s: HB_NS_APPLY_TO_PARAM needs param_step and an output that is not the input", who);
     if ((f & HB_NS_CAUTIOUS_WD) && !(f & HB_NS_APPLY_TO_PARAM)) return set_error(HB_EINVAL, "%s: HB_NS_CAUTIOUS_WD goes with HB_NS_APPLY_TO_PARAM", who);
   }
+  if ((sumsq_parts == nullptr) != (n_sumsq_parts == nullptr)) return set_error(HB_EINVAL, "%s: sumsq_parts and n_sumsq_parts go together", who);
   for (int i = 0; i < n_mats; ++i) {
+    if (sumsq_parts && sumsq_parts[i] && n_sumsq_parts[i] <= 0) return set_error(HB_EINVAL, "%s: no partial sums for matrix %d", who, i);
     if (!g[i] || !out[i]) return set_error(HB_EINVAL, "%s: null matrix pointer at %d", who, i);
     if (rows[i] <= 0 || cols[i] <= 0 || rows[i] > (1 << 20) || cols[i] > (1 << 20)) return set_error(HB_EINVAL, "%s: bad shape at %d", who, i);
   }
@@ -1160,9 +1176,15 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
       q.legacy = (flag_of(i) & HB_NS_LEGACY) != 0;
       q.narrow_update = (flag_of(i) & HB_NS_BF16_UPDATE) ? 1 : (flag_of(i) & HB_NS_F16_UPDATE) ? 2 : 0;
       const int64_t n = p.rows * p.cols;
-      q.n_blocks = (int)std::min<int64_t>(1024, (n + 4095) / 4096);
       q.block_begin = blocks;
-      blocks += q.n_blocks;
+      if (sumsq_parts && sumsq_parts[i]) {  // the caller's partial sums: nothing to launch for this matrix
+        q.partial = sumsq_parts[i];
+        q.n_blocks = n_sumsq_parts[i];
+        q.sum_blocks = 0;
+      } else {
+        q.n_blocks = q.sum_blocks = (int)std::min<int64_t>(1024, (n + 4095) / 4096);
+      }
+      blocks += q.sum_blocks;
       q.tiles_c = (int)((p.cols + 63) / 64);
       q.tile_begin = tiles;
       tiles += (int)((p.rows + 63) / 64) * q.tiles_c;
@@ -1171,8 +1193,8 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
         ns_zero_kernel<<<1024, 256, 0, s>>>(reinterpret_cast<uint4*>(base[i] + p.off_x[0]), n16);
       }
     }
-    ns_sumsq_kernel<<<blocks, 256, 0, s>>>(pg);
-    ns_norm_final_kernel<<<pg.n_items, 256, 0, s>>>(pg);
+    if (blocks > 0) ns_sumsq_kernel<<<blocks, 256, 0, s>>>(pg);
+    ns_norm_final_kernel<<<pg.n_items, kNormThreads, 0, s>>>(pg);
     ns_prep_kernel<<<tiles, 256, 0, s>>>(pg);
   }
 
@@ -1330,7 +1352,7 @@ extern "C" int hb_ns5_batched(int32_t n_mats, const float* const* g, float* cons
                               const float* coeffs_host, int32_t legacy, float eps, const float* post_scale, int32_t rng_mode,
                               uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                               void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, &legacy, false, eps, post_scale, nullptr, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, &legacy, false, eps, post_scale, nullptr, nullptr, nullptr, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched");
 }
 
@@ -1338,21 +1360,23 @@ extern "C" int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float
                                     const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale, int32_t rng_mode,
                                     uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                                     void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, flags, true, eps, post_scale, nullptr, rng_mode, seed, step, flat_base,
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, 5, coeffs_host, flags, true, eps, post_scale, nullptr, nullptr, nullptr, rng_mode, seed, step, flat_base,
                               workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5_batched_mixed");
 }
 
 extern "C" int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                                    int32_t n_steps, const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale,
-                                   const float* param_step, int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base,
-                                   void* workspace, int64_t workspace_bytes, void* stream_) {
-  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, n_steps, coeffs_host, flags, true, eps, post_scale, param_step, rng_mode, seed, step,
-                              flat_base, workspace, workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns_batched_steps");
+                                   const float* param_step, const double* const* sumsq_parts, const int32_t* n_sumsq_parts, int32_t rng_mode,
+                                   uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
+                                   void* stream_) {
+  return hb::ns5_batched_impl(n_mats, g, out, rows, cols, n_steps, coeffs_host, flags, true, eps, post_scale, param_step, sumsq_parts,
+                              n_sumsq_parts, rng_mode, seed, step, flat_base, workspace, workspace_bytes, static_cast<hipStream_t>(stream_),
+                              "hb_ns_batched_steps");
 }
 
 extern "C" int hb_ns5(const float* g, float* out, int64_t rows, int64_t cols, const float* coeffs_host, int32_t legacy, float eps,
                       float post_scale, int32_t rng_mode, uint64_t seed, uint32_t step, int64_t flat_base, void* workspace,
                       int64_t workspace_bytes, void* stream_) {
-  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, 5, coeffs_host, &legacy, false, eps, &post_scale, nullptr, rng_mode, seed, step, &flat_base, workspace,
+  return hb::ns5_batched_impl(1, &g, &out, &rows, &cols, 5, coeffs_host, &legacy, false, eps, &post_scale, nullptr, nullptr, nullptr, rng_mode, seed, step, &flat_base, workspace,
                               workspace_bytes, static_cast<hipStream_t>(stream_), "hb_ns5");
 }

@@ -95,6 +95,14 @@ class Muon(HBOptimizer):
             self._workspace[device] = ws
         return ws
 
+    def _scratch64(self, device, key, n: int) -> torch.Tensor:
+        """A float64 device buffer of at least ``n`` elements that lives as long as the optimizer, one per ``key``."""
+        pool = self.__dict__.setdefault("_scratch64_pool", {})
+        buf = pool.get(key)
+        if buf is None or buf.numel() < n or buf.device != device:
+            buf = pool[key] = torch.empty(max(n, 1), dtype=torch.float64, device=device)
+        return buf
+
     #: upper bound on the Newton-Schulz scratch of one grouped call; a bucket whose matrices need more is split
     ns_workspace_limit = 16 << 30
     #: let the last Newton-Schulz product apply the step to fp32 parameters itself where the chain allows it (same arithmetic as
@@ -207,6 +215,7 @@ class Muon(HBOptimizer):
                 clipped[(id(b), gdt)] = res
         keep = []
         stepped = set()  # (bucket, tensor) whose parameter the last Newton-Schulz product has already updated
+        sumsq = {}  # (bucket, tensor) -> (address, count) of the partial sums of squares the momentum kernel left for it
         tables = {}  # (bucket, gradient dtype) -> device table of gradient pointers
         for b, items, by_dtype in prepared:
             offsets, numel = b.slab.meta()
@@ -225,10 +234,19 @@ class Muon(HBOptimizer):
                     else:  # the clipped gradients live in a slab role
                         g_slab, g_table, g_fmt = clip[0].data_ptr(), None, _PLAIN_FMT[clip[1]]
                     keep.append((table, chunks, lst, clip))
-                    _lib.check(L.hb_momentum(b.slab.ptr(self.KEY), b.slab.ptr(self.KEY + "::ecc"), mom_fmt, b.slab.ptr("_update"), g_slab,
-                                             g_table, g_fmt, offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr(), n_chunks,
-                                             self._mom_mode, a_f, oma_f, self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF, stream),
-                               "hb_momentum")  # fmt: skip
+                    # the momentum kernel leaves the sums of squares of the update it writes, a few doubles per chunk, so that
+                    # Newton-Schulz' norm needs no pass of its own over the update
+                    per_chunk = L.hb_momentum_sumsq_parts_per_chunk()
+                    parts = self._scratch64(b.device, ("sumsq", id(b), gdt), n_chunks * per_chunk)
+                    first = 0
+                    for i in act:
+                        count = -(-b.slab.numels[i] // _lib.chunk_elems())
+                        sumsq[(id(b), i)] = (parts.data_ptr() + 8 * first * per_chunk, count * per_chunk)
+                        first += count
+                    _lib.check(L.hb_momentum_sumsq(b.slab.ptr(self.KEY), b.slab.ptr(self.KEY + "::ecc"), mom_fmt, b.slab.ptr("_update"), g_slab,
+                                                   g_table, g_fmt, offsets.data_ptr(), numel.data_ptr(), chunks.data_ptr(), n_chunks,
+                                                   self._mom_mode, a_f, oma_f, self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF,
+                                                   parts.data_ptr(), stream), "hb_momentum_sumsq")  # fmt: skip
                 # orthogonalise every update with two or more dimensions (heavyball/chainable.py:1117-1126)
                 if mode not in ("newtonschulz", "legacy_newtonschulz", "thinky_polar_express"):
                     # "qr", "svd", "legacy_svd" (heavyball/utils.py:798-806) are factorisations, not this iteration
@@ -266,12 +284,14 @@ class Muon(HBOptimizer):
                     base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
                     arr = (ctypes.c_float * (3 * n_steps * n))(*[x for lg in legacy for x in coeff_tables["polar" if n_steps == 10 else lg]])
                     flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) | tail_flags for (i, _, _), lg in zip(part, legacy)])
+                    ss_ptr = (ctypes.c_void_p * n)(*[sumsq[(id(b), i)][0] for i, _, _ in part])
+                    ss_cnt = (ctypes.c_int32 * n)(*[sumsq[(id(b), i)][1] for i, _, _ in part])
                     nbytes = ctypes.c_int64()
                     _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows_a, cols_a, ctypes.byref(nbytes)))
                     ws = self._ws(b.device, nbytes.value)
-                    _lib.check(L.hb_ns_batched_steps(n, ptrs, outs, rows_a, cols_a, n_steps, arr, flag_a, 1e-7, scale, param_step,
-                                                     self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF, base, ws.data_ptr(),
-                                                     ws.numel(), stream), "hb_ns_batched_steps")  # fmt: skip
+                    _lib.check(L.hb_ns_batched_steps(n, ptrs, outs, rows_a, cols_a, n_steps, arr, flag_a, 1e-7, scale, param_step, ss_ptr,
+                                                     ss_cnt, self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF, base,
+                                                     ws.data_ptr(), ws.numel(), stream), "hb_ns_batched_steps")  # fmt: skip
                 if fuse_tail:
                     stepped.update((id(b), i) for i, _, _ in mats)
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group

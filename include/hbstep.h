@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 10
+#define HB_ABI_VERSION 11
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -238,6 +238,16 @@ int hb_momentum(void* momentum, void* momentum_corr, int32_t momentum_fmt, float
                 const void* const* grad_ptrs, int32_t grad_fmt, const int64_t* offsets, const int64_t* numel,
                 const int32_t* chunks, int64_t n_chunks, int32_t mode, float a, float one_minus_a, int32_t rng_mode,
                 uint64_t seed, uint32_t step, void* stream);
+/* hb_momentum that also leaves the sums of squares of the update it writes, for the norm that Newton-Schulz divides by
+ * (heavyball/utils.py:555) without another pass over the update: sumsq_parts receives
+ * hb_momentum_sumsq_parts_per_chunk() doubles per entry of `chunks`, in the order of `chunks` (zeros past a tensor's end); the
+ * sum over a tensor's chunks is its sum of squares.  Plain stores, no atomics: the same bits in every run.  sumsq_parts
+ * NULL: hb_momentum. */
+int hb_momentum_sumsq_parts_per_chunk(void);
+int hb_momentum_sumsq(void* momentum, void* momentum_corr, int32_t momentum_fmt, float* update, const void* grad,
+                      const void* const* grad_ptrs, int32_t grad_fmt, const int64_t* offsets, const int64_t* numel,
+                      const int32_t* chunks, int64_t n_chunks, int32_t mode, float a, float one_minus_a, int32_t rng_mode,
+                      uint64_t seed, uint32_t step, double* sumsq_parts, void* stream);
 
 /*
  * hb_ns5 replaces zeropower_via_newtonschulz5 (heavyball/utils.py:550-577; legacy != 0: legacy_zeropower_via_newtonschulz5,
@@ -294,11 +304,15 @@ int hb_ns5_batched_mixed(int32_t n_mats, const float* const* g, float* const* ou
  * PARAMETER (not g[i]) and takes p <- p * param_step[0] + update * param_step[1], i.e. update_param_ without caution
  * (heavyball/utils.py:2373-2406) with param_step = {1 - decay * lr, -lr} in HOST memory, in the arithmetic of hb_update_param;
  * the update itself is not written anywhere.  HB_NS_CAUTIOUS_WD with it: the first factor is 1 where update and parameter
- * differ in sign (cautious weight decay). */
+ * differ in sign (cautious weight decay).
+ * sumsq_parts / n_sumsq_parts (HOST arrays of n_mats entries, or both NULL): where sumsq_parts[i] is not NULL it points to
+ * n_sumsq_parts[i] doubles in DEVICE memory whose sum is the sum of squares of g[i] (hb_momentum_sumsq leaves them), and the
+ * call does not read g[i] a first time to compute its norm. */
 int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out, const int64_t* rows, const int64_t* cols,
                         int32_t n_steps, const float* coeffs_host, const int32_t* flags, float eps, const float* post_scale,
-                        const float* param_step, int32_t rng_mode, uint64_t seed, uint32_t step, const int64_t* flat_base,
-                        void* workspace, int64_t workspace_bytes, void* stream);
+                        const float* param_step, const double* const* sumsq_parts, const int32_t* n_sumsq_parts, int32_t rng_mode,
+                        uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
+                        void* stream);
 
 /* Test hook: ONE product of the Newton-Schulz iteration on bf16 operands (row-major, K contiguous: A [M, K], B [N, K]) through
  * the kernel of the given tile class (128 or 256), so that a test can put the same product through both kernels, whose

@@ -267,7 +267,8 @@ def run_ns_steps(Gs, coeffs, rng_mode=_lib.RNG_HALF, seed=0, step=0, bases=None)
     op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
     scale = (ctypes.c_float * n)(*[1.0] * n)
     base = (ctypes.c_int64 * n)(*(bases or [0] * n))
-    _lib.check(L.hb_ns_batched_steps(n, gp, op, rows, cols, n_steps, arr, flags, 1e-7, scale, None, rng_mode, seed, step, base, ws.data_ptr(), nbytes.value, None),
+    _lib.check(L.hb_ns_batched_steps(n, gp, op, rows, cols, n_steps, arr, flags, 1e-7, scale, None, None, None, rng_mode, seed, step, base, ws.data_ptr(),
+                                     nbytes.value, None),
                "hb_ns_batched_steps")  # fmt: skip
     torch.cuda.synchronize()
     return [o.cpu() for o in outs]
@@ -519,6 +520,41 @@ def test_step_inside_the_last_product_equals_the_separate_update(kwargs, gdt):
         for i, (p, q) in enumerate(zip(pa, pb)):
             assert torch.equal(p.detach().view(torch.int32), q.detach().view(torch.int32)), (k, i, shapes[i])
     assert all(not torch.equal(p.detach().cpu(), h) for p, h in zip(pa, host))  # and they did move
+
+
+def test_momentum_leaves_the_sums_of_squares_of_its_update():
+    """hb_momentum_sumsq: the doubles it writes per chunk add up, tensor by tensor, to the sum of squares of the update it wrote
+    (ragged sizes: a chunk's tail past the tensor's end contributes zeros), for fp32 and for bf16 gradients, whose update is
+    rounded before it is squared.  Read off a Muon step whose last product applies the parameter step itself, so the update
+    buffer still holds what the momentum kernel wrote."""
+    import heavyball_amd
+    from tests import helpers as H
+
+    shapes = [(192, 320), (4097,), (130, 70), (1, 5), (8, 6, 24), (1100, 1024)]
+    L = _lib.lib()
+    per_chunk, chunk = L.hb_momentum_sumsq_parts_per_chunk(), _lib.chunk_elems()
+    for gdt in (torch.float32, torch.bfloat16):
+        print("case", gdt, flush=True)
+        _, params = H.make_params(shapes, DEV)
+        opt = heavyball_amd.Muon(params, lr=0.02)
+        for p, g in zip(params, H.make_grads(shapes, 1, gdt, 1e-2)):
+            p.grad = g.to(DEV)
+        opt.step()
+        torch.cuda.synchronize()
+        (b,) = opt._buckets[0]
+        parts = opt._scratch64_pool[("sumsq", id(b), gdt)].cpu()
+        first = 0
+        for i, n in enumerate(b.slab.numels):
+            count = -(-n // chunk)
+            got = parts[first * per_chunk : (first + count) * per_chunk]
+            first += count
+            u = b.slab.view("_update", i).double().cpu()
+            assert u.abs().max() > 0
+            if gdt == torch.bfloat16:
+                assert torch.equal(u, u.bfloat16().double())
+            want = (u * u).sum()
+            assert abs(got.sum() - want) <= 1e-12 * want, (i, float(got.sum()), float(want))
+            assert (got >= 0).all()
 
 
 def _random_muon_case(seed):
