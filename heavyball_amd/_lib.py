@@ -103,6 +103,7 @@ _PROTOTYPES = {
     "hb_ns_batched_steps": (ctypes.c_int, [c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64), c_int32, POINTER(c_float),
                                            POINTER(c_int32), c_float, POINTER(c_float), POINTER(c_float), POINTER(c_void_p), POINTER(c_int32),
                                            c_int32, c_uint64, c_uint32, POINTER(c_int64), c_void_p, c_int64, c_void_p]),
+    "hb_ns_tile": (ctypes.c_int, [c_int64, c_int64]),
     "hb_ns_product": (ctypes.c_int, [c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_void_p,
                                      c_int64, c_void_p]),
     "hb_ns5": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_int64, POINTER(c_float), c_int32, c_float, c_float, c_int32, c_uint64, c_uint32,

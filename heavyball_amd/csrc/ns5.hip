@@ -34,7 +34,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 
-enum { kModeS = 0, kModeY2 = 1, kModeX = 2, kModeFinal = 3, kModePartial = 4 };  // kModePartial: raw fp32 product of one K chunk
+// kModePartial: raw fp32 product of one K chunk.  kModeFinalX: kModeFinal with the rarer epilogues (a float16 update buffer, the
+// parameter step applied in place); they live in a kernel of their own so that the common last product stays as small as it was
+// (with them inside, the 256-wide kernel's plain last product took 11 % longer).
+enum { kModeS = 0, kModeY2 = 1, kModeX = 2, kModeFinal = 3, kModePartial = 4, kModeFinalX = 5 };
 
 // One entry of a grouped launch: a run of consecutive tiles of one matrix, on one XCD (see locate_tile).  A launch multiplies
 // any number of independent matrices.
@@ -256,9 +259,9 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
       // chain (heavyball/utils.py:2373-2390; the two factors travel in mul_c and diag, which this mode has no other use for), with
       // the decay factor 1 where update and parameter disagree in sign under kCautiousWd.  The sub-tile's 16 parameter values
       // are read before any of them is written, so that the loads are in flight together.
-      const bool apply = MODE == kModeFinal && (g.round_out & kApplyToParam) != 0;
+      const bool apply = MODE == kModeFinalX && (g.round_out & kApplyToParam) != 0;
       float pv[16];
-      if (MODE == kModeFinal && apply) {
+      if (MODE == kModeFinalX && apply) {
 #pragma unroll
         for (int rb4 = 0; rb4 < 4; ++rb4) {
           const int row = row_tile + rb4 * 8 + erow;
@@ -285,7 +288,7 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
 #pragma unroll
       for (int rb4 = 0; rb4 < 4; ++rb4) {
         const int row = row_tile + rb4 * 8 + erow;
-        if (MODE == kModeFinal || MODE == kModePartial) {
+        if (MODE == kModeFinal || MODE == kModeFinalX || MODE == kModePartial) {
           float o[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
@@ -294,11 +297,11 @@ __device__ __forceinline__ void ns_epilogue(floatx16 (&acc)[TM][TN], const Probl
             } else {
               o[r] = bf16_to_f32(prim[rb4 * 4 + r]) * g.scale;  // x.to(G.dtype) then y *= scale (heavyball/utils.py:577, :808-809)
               if ((g.round_out & 3) == 1) o[r] = bf16_to_f32(f32_to_bf16_rne(o[r]));  // ... in bf16 when G is bf16
-              else if ((g.round_out & 3) == 2)  // fp16: the cast leaves bf16's range (subnormals, overflow), then the product rounds again
+              else if (MODE == kModeFinalX && (g.round_out & 3) == 2)  // fp16: the cast leaves bf16's range (subnormals, overflow), then the product rounds again
                 o[r] = f16_to_f32(f32_to_f16_rne(f16_to_f32(f32_to_f16_rne_plain(bf16_to_f32(prim[rb4 * 4 + r]))) * g.scale));
             }
           }
-          if (MODE == kModeFinal && apply) {
+          if (MODE == kModeFinalX && apply) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[r] = stepped(pv[rb4 * 4 + r], o[r]);
           }
@@ -1292,7 +1295,12 @@ static int ns5_batched_impl(int n_mats, const float* const* g, float* const* out
           probs[k] = q;
         }
         if (it < n_steps - 1) gemm_stage<kModeX>(st, probs, t, s);
-        else gemm_stage<kModeFinal>(st, probs, t, s);
+        else {
+          bool extras = false;  // anything the plain last product does not do: see kModeFinalX
+          for (const Problem& q : probs) extras = extras || (q.round_out & ~1) != 0;
+          if (extras) gemm_stage<kModeFinalX>(st, probs, t, s);
+          else gemm_stage<kModeFinal>(st, probs, t, s);
+        }
       }
     }
     if (int rc = run_staged(st, dev_tables, table_room, s, who)) return rc;
@@ -1342,6 +1350,12 @@ extern "C" int hb_ns_product(int32_t tile, int32_t mode, const void* A, const vo
   else if (mode == kModeY2) gemm_stage<kModeY2>(st, {q}, tile, s);
   else gemm_stage<kModeX>(st, {q}, tile, s);
   return run_staged(st, static_cast<char*>(workspace), 4096, s, "hb_ns_product");
+}
+
+extern "C" int hb_ns_tile(int64_t rows, int64_t cols) {
+  std::vector<int> tile;
+  hb::choose_tiles(1, &rows, &cols, tile);
+  return tile[0];
 }
 
 extern "C" int hb_ns5_workspace_bytes(int64_t rows, int64_t cols, int64_t* bytes) {

@@ -259,11 +259,14 @@ class Muon(HBOptimizer):
                 ns_flags = {i: _NS_UPDATE_FLAG[gdt] for gdt, lst in by_dtype.items() for i, _ in lst}
                 # an fp32 parameter that nothing else looks at between Newton-Schulz and update_param_ (no caution, whose mask needs
                 # the finished update of the whole tensor, and no clip of the update) takes its step in the epilogue of the last
-                # product: the update is never written out and read back
+                # product: the update is never written out and read back.  Matrices of the 128-wide kernel only: the 256-wide one
+                # runs a single workgroup per compute unit, and the longer epilogue costs more there than the pass it saves.
                 fuse_tail = (self.fuse_update_into_newton_schulz and not group["caution"] and self.update_clipping is None and not pecc
                              and b.param_dtype == torch.float32)  # fmt: skip
                 tail_flags = (_lib.NS_APPLY_TO_PARAM | (_lib.NS_CAUTIOUS_WD if flags & _lib.FLAG_CAUTIOUS_WD else 0)) if fuse_tail else 0
                 param_step = (ctypes.c_float * 2)(omdl, neg_lr)
+                fused = {i for i, r, c in ((i, p.shape[0], p.numel() // p.shape[0]) for i, p, _ in items if p.dim() >= 2)
+                         if fuse_tail and L.hb_ns_tile(r, c) == 128}  # fmt: skip
                 mats = []
                 for i, p, _ in items:
                     if p.dim() < 2:
@@ -279,11 +282,12 @@ class Muon(HBOptimizer):
                     rows_a = (ctypes.c_int64 * n)(*[r for _, r, _ in part])
                     cols_a = (ctypes.c_int64 * n)(*[c for _, _, c in part])
                     ptrs = (ctypes.c_void_p * n)(*[b.slab.view("_update", i).data_ptr() for i, _, _ in part])
-                    outs = (ctypes.c_void_p * n)(*[b.slab.view("param", i).data_ptr() for i, _, _ in part]) if fuse_tail else ptrs
+                    outs = (ctypes.c_void_p * n)(*[b.slab.view("param" if i in fused else "_update", i).data_ptr() for i, _, _ in part])
                     scale = (ctypes.c_float * n)(*[max(1, r / c) ** 0.5 for _, r, c in part])  # heavyball/utils.py:808-809
                     base = (ctypes.c_int64 * n)(*[int(b.slab.offsets_np[i]) for i, _, _ in part])
                     arr = (ctypes.c_float * (3 * n_steps * n))(*[x for lg in legacy for x in coeff_tables["polar" if n_steps == 10 else lg]])
-                    flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) | tail_flags for (i, _, _), lg in zip(part, legacy)])
+                    flag_a = (ctypes.c_int32 * n)(*[ns_flags[i] | int(lg) | (tail_flags if i in fused else 0)
+                                                    for (i, _, _), lg in zip(part, legacy)])  # fmt: skip
                     ss_ptr = (ctypes.c_void_p * n)(*[sumsq[(id(b), i)][0] for i, _, _ in part])
                     ss_cnt = (ctypes.c_int32 * n)(*[sumsq[(id(b), i)][1] for i, _, _ in part])
                     nbytes = ctypes.c_int64()
@@ -292,8 +296,7 @@ class Muon(HBOptimizer):
                     _lib.check(L.hb_ns_batched_steps(n, ptrs, outs, rows_a, cols_a, n_steps, arr, flag_a, 1e-7, scale, param_step, ss_ptr,
                                                      ss_cnt, self._rng_mode(), self.rng_seed, int(step) & 0xFFFFFFFF, base,
                                                      ws.data_ptr(), ws.numel(), stream), "hb_ns_batched_steps")  # fmt: skip
-                if fuse_tail:
-                    stepped.update((id(b), i) for i, _, _ in mats)
+                stepped.update((id(b), i) for i in fused)
         if self.update_clipping is not None:  # heavyball/chainable.py:2700-2701: on the finished update of the whole group
             keep.append((yield (self.update_clipping, "_update", [(b, sorted(i for i, _, _ in items)) for b, items, _ in prepared])))
             for b, items, by_dtype in prepared:

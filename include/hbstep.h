@@ -314,6 +314,11 @@ int hb_ns_batched_steps(int32_t n_mats, const float* const* g, float* const* out
                         uint64_t seed, uint32_t step, const int64_t* flat_base, void* workspace, int64_t workspace_bytes,
                         void* stream);
 
+/* The tile width (128 or 256) of the product kernel that a rows x cols matrix goes through.  The wide kernel runs one workgroup
+ * per compute unit, with nothing to hide an epilogue behind: HB_NS_APPLY_TO_PARAM costs more there than the separate
+ * hb_update_param it saves, so a caller asks first. */
+int hb_ns_tile(int64_t rows, int64_t cols);
+
 /* Test hook: ONE product of the Newton-Schulz iteration on bf16 operands (row-major, K contiguous: A [M, K], B [N, K]) through
  * the kernel of the given tile class (128 or 256), so that a test can put the same product through both kernels, whose
  * accumulation order is the same and whose results must agree bit for bit.  mode 0: C = bf16(A B^T), C2 = bf16(bf16(C * mul_c) +

@@ -274,6 +274,56 @@ def run_ns_steps(Gs, coeffs, rng_mode=_lib.RNG_HALF, seed=0, step=0, bases=None)
     return [o.cpu() for o in outs]
 
 
+@pytest.mark.parametrize("cautious", [False, True])
+def test_apply_to_param_equals_the_product_followed_by_the_update(cautious):
+    """HB_NS_APPLY_TO_PARAM through the C ABI, on both product kernels (tall, wide and ragged matrices of the 128- and the 256-wide
+    class, fp32 and float16 update buffers): the parameter ends where the plain call's update, put through
+    p * (1 - decay lr) + u * (-lr) in fp32 (decay factor 1 where signs differ under HB_NS_CAUTIOUS_WD), puts it, bit for bit;
+    the update buffer handed in is left alone."""
+    L = _lib.lib()
+    gen = torch.Generator().manual_seed(29)
+    shapes = [(320, 192), (130, 515), (1100, 1024), (1024, 1280)]
+    Gs = [torch.randn(s, generator=gen) * 1e-2 for s in shapes]
+    Gs[1] = Gs[1].half().float()
+    Ps = [torch.randn(s, generator=gen) * 0.05 for s in shapes]
+    n = len(Gs)
+    rows = (ctypes.c_int64 * n)(*[g.shape[0] for g in Gs])
+    cols = (ctypes.c_int64 * n)(*[g.shape[1] for g in Gs])
+    assert [L.hb_ns_tile(*s) for s in shapes] == [128, 128, 256, 256]
+    nbytes = ctypes.c_int64()
+    _lib.check(L.hb_ns5_batched_workspace_bytes(n, rows, cols, ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
+    gs = [g.to(DEV).contiguous() for g in Gs]
+    us = [torch.empty_like(g) for g in gs]
+    ps = [p.to(DEV).contiguous() for p in Ps]
+    arr = (ctypes.c_float * (15 * n))(*(ns_coeff_array(muon.NS_COEFFS) * n))
+    base_flags = [0, _lib.NS_F16_UPDATE, 0, 0]
+    scale = (ctypes.c_float * n)(*[max(1, g.shape[0] / g.shape[1]) ** 0.5 for g in Gs])
+    base = (ctypes.c_int64 * n)(*[4096 * 300 * k for k in range(n)])
+    gp = (ctypes.c_void_p * n)(*[g.data_ptr() for g in gs])
+    om, neg_lr = 1 - 0.1 * 0.02, -0.02
+    step = (ctypes.c_float * 2)(om, neg_lr)
+
+    def call(outs, extra):
+        flags = (ctypes.c_int32 * n)(*[f | extra for f in base_flags])
+        op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+        _lib.check(L.hb_ns_batched_steps(n, gp, op, rows, cols, 5, arr, flags, 1e-7, scale, step, None, None, _lib.RNG_PHILOX, 5, 3, base,
+                                         ws.data_ptr(), nbytes.value, None), "hb_ns_batched_steps")  # fmt: skip
+        torch.cuda.synchronize()
+
+    print("case", cautious, flush=True)
+    call(us, 0)
+    call(ps, _lib.NS_APPLY_TO_PARAM | (_lib.NS_CAUTIOUS_WD if cautious else 0))
+    for k in range(n):
+        p0, u = Ps[k].to(DEV), us[k]
+        factor = torch.full_like(p0, om)
+        if cautious:
+            factor = torch.where((p0.view(torch.int32) ^ u.view(torch.int32)) < 0, torch.ones_like(p0), factor)
+        want = p0 * factor + u * torch.tensor(neg_lr, dtype=torch.float32, device=DEV)
+        assert torch.equal(ps[k].view(torch.int32), want.view(torch.int32)), shapes[k]
+        assert torch.equal(gs[k].cpu(), Gs[k])
+
+
 def test_polar_express_matches_reference_vectors_and_oracle():
     """hb_ns_batched_steps under msign's ten-step schedule: against the vectors the reference computed (fp32, bf16 and float16
     inputs, one call for all five), against the oracle on larger matrices of both tile classes, and with five steps of the default
@@ -530,7 +580,7 @@ def test_momentum_leaves_the_sums_of_squares_of_its_update():
     import heavyball_amd
     from tests import helpers as H
 
-    shapes = [(192, 320), (4097,), (130, 70), (1, 5), (8, 6, 24), (1100, 1024)]
+    shapes = [(192, 320), (4097,), (130, 70), (1, 5), (8, 6, 24), (700, 900)]  # matrices of the 128-wide kernel: the step is fused
     L = _lib.lib()
     per_chunk, chunk = L.hb_momentum_sumsq_parts_per_chunk(), _lib.chunk_elems()
     for gdt in (torch.float32, torch.bfloat16):
