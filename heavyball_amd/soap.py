@@ -340,7 +340,7 @@ class SOAP(HBOptimizer):
             b.slab.role("_update", torch.float32)
             gemm = _Gemm(b.device)
             stream = current_stream_ptr(b.device)
-            updated, keep, refresh = [], [], []
+            updated, keep, refresh, first = [], [], [], []
             with torch.cuda.device(b.device):
                 def precondition(st, G0, G, out, base, fdt):
                     """One tensor or block: G0 the gradient, G the update that goes through the preconditioner, both in the merged
@@ -362,7 +362,8 @@ class SOAP(HBOptimizer):
                             # 16-bit factors: the first one is the rounded product itself (the reference's contraction of a 16-bit
                             # gradient returns that dtype, utils.py:1387); the basis below comes from the stored values and is cast (:1003)
                             GG = [None if m is None else m.to(fdt) for m in GG]
-                        st[K_GG], st[K_Q] = GG, self._first_bases(G0, GG, fdt, base)
+                        st[K_GG] = GG
+                        first.append((st, G0, GG, fdt, base))  # the bases of every tensor's first step are found together, below
                         st.setdefault("is_initialized", set()).update({0, 2, 3})
                         return False
                     GG, Q = self._factors32(st)
@@ -427,6 +428,9 @@ class SOAP(HBOptimizer):
                         start += gb.numel()
                     if done:
                         updated.append(i)
+                if first:
+                    for (st, *_), Q in zip(first, self._first_bases_of([e[1:] for e in first])):
+                        st[K_Q] = Q
                 if refresh:
                     self._refresh(gemm, refresh)
                     for GG32, Q32, exp_avg, st, base in refresh:
@@ -616,7 +620,12 @@ class SOAP(HBOptimizer):
         return torch.flip(vec, [-1])
 
     def _first_bases(self, G0, GG, fdt, seed_base: int):
-        """The eigenbases of the first factors (heavyball/utils.py:986-1038).
+        """The eigenbases of one tensor's first factors: ``_first_bases_of`` for a single entry."""
+        return self._first_bases_of([(G0, GG, fdt, seed_base)])[0]
+
+    def _first_bases_of(self, entries):
+        """The eigenbases of the first factors (heavyball/utils.py:986-1038) of ``entries`` = [(G0, GG, fdt, seed_base), ...], the
+        tensors (or blocks) that take their first step in this call; one list of bases per entry.
 
         A matrix gradient G with both factors takes one eigensolve, on its smaller side: the first factors are G G^T and G^T G,
         so the eigenvectors of one are the singular vectors of G on that side and the other side's follow as G^T U (or G U)
@@ -625,28 +634,50 @@ class SOAP(HBOptimizer):
         completion is an eigenbasis to that accuracy, and a seeded random one is taken.  ``hb_orthonormalize_f32`` then makes the
         whole basis orthonormal to fp32 (its first columns already are, and stay).  An 8192-wide factor of a 2048 x 8192 gradient
         costs 37 ms this way instead of a 670 ms eigensolve.  Everything else (factors kept in 16 bits, whose stored values are
-        no exact product any more; views with more than two dimensions; a single factor) takes the eigensolver per factor."""
-        Q: List[Optional[torch.Tensor]] = [None] * len(GG)
-        paired = fdt == torch.float32 and G0.dim() == 2 and len(GG) == 2 and GG[0] is not None and GG[1] is not None
-        done = set()
-        if paired:
-            s = 0 if G0.shape[0] <= G0.shape[1] else 1  # the smaller side
-            U = self._eigh_basis(GG[s][0])
-            W = (G0.T if s == 0 else G0).double() @ U  # [larger, smaller]: unnormalised singular vectors of the other side
-            norms = W.norm(dim=0)
-            good = norms > 1e-6 * norms.max()  # a column below that belongs to the null space of G itself
-            gen = torch.Generator(device=G0.device)
-            gen.manual_seed(0x50A9 + int(seed_base))  # the tensor's place in its slab: the same completion in every run
-            big, small = W.shape
-            other = torch.randn(big, big, device=G0.device, dtype=torch.float32, generator=gen)
-            other[:, :small] = torch.where(good, (W / norms.clamp(min=1e-300)).float(), other[:, :small])
-            if orthonormalize_(other):
-                Q[s], Q[1 - s] = U.to(fdt).contiguous()[None], other[None]
-                done = {0, 1}
-        for d, m in enumerate(GG):
-            if m is not None and d not in done:
-                Q[d] = self._eigh_basis(m).to(fdt).contiguous()
-        return Q
+        no exact product any more; views with more than two dimensions; a single factor) takes the eigensolver per factor.
+
+        The eigensolves of one width go to the solver as one batch: below a few thousand columns a solve is a long chain of small
+        kernels, and a batch runs the chains of all its matrices side by side (twelve 768-wide factors: 27 ms instead of 216)."""
+        def is_paired(G0, GG, fdt):
+            return fdt == torch.float32 and G0.dim() == 2 and len(GG) == 2 and GG[0] is not None and GG[1] is not None
+
+        wanted: Dict[tuple, List] = {}  # (device, width) -> [((entry, side), factor)]
+        for e, (G0, GG, fdt, _) in enumerate(entries):
+            if is_paired(G0, GG, fdt):
+                sides = [0 if G0.shape[0] <= G0.shape[1] else 1]  # the smaller side
+            else:
+                sides = [d for d, m in enumerate(GG) if m is not None]
+            for d in sides:
+                wanted.setdefault((GG[d].device, GG[d].shape[-1]), []).append(((e, d), GG[d][0]))
+        solved = {}
+        for (_, n), lst in wanted.items():
+            per = max(1, (1 << 30) // (8 * n * n))  # stacks of at most 1 GiB of float64
+            for k in range(0, len(lst), per):
+                part = lst[k : k + per]
+                for (key, _), vec in zip(part, self._eigh_basis(torch.stack([m for _, m in part]))):
+                    solved[key] = vec
+        out = []
+        for e, (G0, GG, fdt, seed_base) in enumerate(entries):
+            Q: List[Optional[torch.Tensor]] = [None] * len(GG)
+            if is_paired(G0, GG, fdt):
+                s = 0 if G0.shape[0] <= G0.shape[1] else 1
+                U = solved[(e, s)]
+                W = (G0.T if s == 0 else G0).double() @ U  # [larger, smaller]: unnormalised singular vectors of the other side
+                norms = W.norm(dim=0)
+                good = norms > 1e-6 * norms.max()  # a column below that belongs to the null space of G itself
+                gen = torch.Generator(device=G0.device)
+                gen.manual_seed(0x50A9 + int(seed_base))  # the tensor's place in its slab: the same completion in every run
+                big, small = W.shape
+                other = torch.randn(big, big, device=G0.device, dtype=torch.float32, generator=gen)
+                other[:, :small] = torch.where(good, (W / norms.clamp(min=1e-300)).float(), other[:, :small])
+                Q[s] = U.to(fdt).contiguous()[None]
+                Q[1 - s] = other[None] if orthonormalize_(other) else self._eigh_basis(GG[1 - s]).to(fdt).contiguous()
+            else:
+                for d, m in enumerate(GG):
+                    if m is not None:
+                        Q[d] = solved[(e, d)].to(fdt).contiguous()[None]
+            out.append(Q)
+        return out
 
     @staticmethod
     def _update_ggt(gemm, G, GG, a: float, one_minus_a: float):

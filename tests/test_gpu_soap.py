@@ -372,6 +372,41 @@ def test_soap_first_bases_from_one_eigensolve(shape, kind):
     assert all(torch.equal(a, b) for a, b in zip(Q, Q2))
 
 
+def test_soap_first_bases_of_several_tensors_are_found_together():
+    """The first step's eigensolves of one width go to the solver as one batch, across the tensors of the step: a first step over
+    matrices that share their smaller side (and one that does not, one with a 16-bit gradient, whose factors take a solve each,
+    and a stack with three factors) leaves every basis orthonormal and diagonalising its stored factor; and the step that
+    follows moves every parameter."""
+    shapes = [(96, 256), (300, 96), (96, 96), (64, 200), (6, 40, 50), (33,)]
+    gen = torch.Generator().manual_seed(5)
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(DEV)) for s in shapes]
+    for p in params:
+        p.grad_dtype = None
+    opt = heavyball_amd.SOAP(params, max_precond_dim=512, precondition_frequency=3)
+    for k in range(2):
+        for i, p in enumerate(params):
+            g = torch.randn(p.shape, generator=gen) * 1e-2
+            p.grad = (g.bfloat16() if i == 3 else g).to(DEV)
+        before = [p.detach().clone() for p in params]
+        opt.step()
+    torch.cuda.synchronize()
+    assert all(not torch.equal(a, p.detach()) for a, p in zip(before, params))
+    widths = []
+    for i, p in enumerate(params):
+        st = opt.state[p][0]
+        for q, gg in zip(st["scale_by_soap_Q_3"], st["scale_by_soap_GG_3"]):
+            if q is None:
+                assert gg is None
+                continue
+            assert q.dtype == gg.dtype == (torch.bfloat16 if i == 3 else torch.float32)
+            widths.append(q.shape[-1])
+            q, gg = q[0].double(), gg[0].double()
+            d = q.shape[0]
+            tol = 2e-2 if i == 3 else 5e-6  # a basis stored in bf16 is orthonormal to bf16
+            assert (q.T @ q - torch.eye(d, device=DEV, dtype=torch.float64)).abs().max().item() < tol, (i, d)
+    assert sorted(widths) == sorted([96, 256, 300, 96, 96, 96, 64, 200, 6, 40, 50])
+
+
 def test_soap_mid_size_own_eigh_signed_momentum():
     """[256, 256] and [512, 512] Gaussian gradients with the optimizer's own eigh (no basis adopted) over two refreshes:
     square gradients give full-rank factors from the first step on, so the eigenbasis is unique up to column signs, and
