@@ -424,6 +424,46 @@ def bench_soap_default_dim(steps=12):
             "refresh_step_ms": round(min(refresh), 3) if refresh else None, "algorithmic_flops_per_step": 515396075520}  # fmt: skip
 
 
+def bench_soap_gpt2(steps=30):
+    """SOAP with the default max_precond_dim on the headline parameter set: 49 matrices of 768 rows, 61 factors of 768 columns (the
+    wider sides exceed max_precond_dim = 2048 and go without), 98 vectors through Adam.  The per-tensor products are mid-sized
+    (108 tiles for a 768 x 2304 projection) and share launches across tensors; ``one_tensor_at_a_time`` is the same step with
+    that switched off."""
+    import torch
+
+    import heavyball_amd
+
+    dev = torch.device("cuda:0")
+    shapes = gpt2_small_shapes()
+    out = {"workload": "SOAP max_precond_dim 2048 (the default), precondition_frequency 10, GPT-2-small-shaped 147 tensors, fp32"}
+    for key, grouped in (("ms_per_step", True), ("one_tensor_at_a_time_ms_per_step", False)):
+        torch.manual_seed(5)
+        params = [torch.nn.Parameter(torch.randn(s, device=dev) * 0.02) for s in shapes]
+        opt = heavyball_amd.SOAP(params, precondition_frequency=10)  # as in the C5 leg: a refresh every 10th step
+        opt.group_products = grouped
+        grad_sets = [[torch.randn(s, device=dev) * 1e-2 for s in shapes] for _ in range(3)]
+        plain, refresh = [], []
+        for k in range(steps + 2):
+            for p, g in zip(params, grad_sets[k % 3]):
+                p.grad = g
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            opt.step()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3
+            if k == 0 and grouped:
+                out["init_step_ms"] = round(ms, 1)
+            elif k >= 2:
+                (refresh if opt.param_groups[0]["is_preconditioning"] else plain).append(ms)
+        plain.sort()
+        out[key] = round(plain[len(plain) // 2], 3)
+        if grouped:
+            out["refresh_step_ms"] = round(min(refresh), 3) if refresh else None
+        del opt, params, grad_sets
+        torch.cuda.empty_cache()
+    return out
+
+
 def bench_soap_products(reps=3):
     """The 18 products of one SOAP step of configuration 5 on random operands, without an optimizer around them (no eigh,
     no basis refresh): a short run of a few dozen launches, meant for hardware-counter collection on the fp32 GEMM kernels.
@@ -640,6 +680,8 @@ def main():
         out["soap"] = bench_soap()
         torch.cuda.empty_cache()
         out["soap"]["default_max_precond_dim"] = bench_soap_default_dim()
+        torch.cuda.empty_cache()
+        out["soap_gpt2"] = bench_soap_gpt2()
     if args.config == "c2" and not args.no_8b:
         # the 8B-shaped parameter set (benchmark configuration 3), under the headline's optimizer and under its own
         torch.cuda.empty_cache()

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("HBSTEP_LIB") or os.path.join(_HERE, "libhbstep.so")
 
 # include/hbstep.h
-ABI_VERSION = 11  # HB_ABI_VERSION this binding was written against
+ABI_VERSION = 12  # HB_ABI_VERSION this binding was written against
 FMT_F32, FMT_BF16, FMT_F16, FMT_ECC_BF16_8, FMT_ECC_BF16_16, FMT_ECC_F16_8, FMT_ECC_F16_16 = range(7)
 ALGO_ADAM, ALGO_LAPROP, ALGO_ADOPT, ALGO_ADEMAMIX, ALGO_NADAM = range(5)
 FLAG_MARS, FLAG_CAUTION, FLAG_CAUTIOUS_WD, FLAG_WRITE_GRAD, FLAG_UPDATE_ONLY, FLAG_ADOPT_WARMUP, FLAG_COUPLED_WD, FLAG_MARS_ONLY = 1, 2, 4, 8, 16, 32, 64, 128
@@ -110,6 +110,9 @@ _PROTOTYPES = {
                               c_int64, c_void_p, c_int64, c_void_p]),
     "hb_gemm_f32": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32,
                                    c_float, c_float, c_void_p]),
+    "hb_gemm_f32_grouped": (ctypes.c_int, [c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64),
+                                           POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int32, c_int32, POINTER(c_int32),
+                                           POINTER(c_float), POINTER(c_float), c_void_p]),
     "hb_orthonormalize_workspace_bytes": (ctypes.c_int, [c_int64, c_int64, POINTER(c_int64)]),
     "hb_orthonormalize_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "hb_orthonormalize_f32_batched": (ctypes.c_int, [c_int32, POINTER(c_void_p), c_int64, c_int64, c_int64, POINTER(c_void_p), c_int64,

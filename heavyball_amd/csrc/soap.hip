@@ -196,24 +196,17 @@ __device__ __forceinline__ void sgemm_mainloop(const SgemmArgs& g, float (*As)[k
 #undef HB_SG_STORE
 }
 
+// One 128 x 128 tile of one product: workgroup `tile` of the problem's grid, k chunk `split` of a split-K launch.
 // TA: A is given as [K, M] (op(A) = A^T); TB: B is given as [N, K] (op(B) = B^T)
 template <bool TA, bool TB>
-__global__ __launch_bounds__(kGThreads, 3) void sgemm_kernel(const SgemmArgs g0, const Batch bt, const unsigned where) {
-  SgemmArgs g = g0;
-  if (bt.n > 1) {
-    const int z = blockIdx.z;
-    g.A = shifted(g0.A, where & kAInWs ? bt.dws[z] : bt.dq[z]);
-    g.B = shifted(g0.B, where & kBInWs ? bt.dws[z] : bt.dq[z]);
-    g.C = shifted(g0.C, where & kCInWs ? bt.dws[z] : bt.dq[z]);
-    if (g0.part) g.part = shifted(g0.part, bt.dws[z]);
-  }
+__device__ __forceinline__ void sgemm_tile(const SgemmArgs& g, const int tile, const int split) {
   __shared__ __attribute__((aligned(16))) float As[2][kGK * kGLD];
   __shared__ __attribute__((aligned(16))) float Bs[2][kGK * kGLD];
   const int tiles_n = (g.N + kGN - 1) / kGN;
-  int bi = blockIdx.x / tiles_n, bj = blockIdx.x % tiles_n;
+  int bi = tile / tiles_n, bj = tile % tiles_n;
   bool mirror = false;
   if (g.sym) {  // workgroups 3d, 3d+1, 3d+2: tiles (2d, 2d), (2d, 2d+1) and (2d+1, 2d+1) of diagonal block d
-    const int d = blockIdx.x / 3, w = blockIdx.x % 3;
+    const int d = tile / 3, w = tile % 3;
     bi = 2 * d + (w == 2);
     bj = 2 * d + (w >= 1);
     mirror = w == 1;
@@ -230,7 +223,7 @@ __global__ __launch_bounds__(kGThreads, 3) void sgemm_kernel(const SgemmArgs g0,
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const int kb = g.part ? blockIdx.y * g.k_chunk : 0;
+  const int kb = g.part ? split * g.k_chunk : 0;
   const int ke = g.part ? (kb + g.k_chunk < g.K ? kb + g.k_chunk : g.K) : g.K;
   const bool interior = row0 + kGM <= g.M && col0 + kGN <= g.N && (ke - kb) % kGK == 0 && kb % 4 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 &&
                         ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0;
@@ -250,7 +243,7 @@ __global__ __launch_bounds__(kGThreads, 3) void sgemm_kernel(const SgemmArgs g0,
         if (row >= g.M) continue;
         const float v = acc[i][j][r];
         if (g.part) {  // split-K: the epilogue runs in splitk_reduce_kernel
-          g.part[((size_t)blockIdx.y * g.M + row) * g.N + col] = v;
+          g.part[((size_t)split * g.M + row) * g.N + col] = v;
           continue;
         }
         float* c = g.C + (size_t)row * g.ldc + col;
@@ -260,6 +253,48 @@ __global__ __launch_bounds__(kGThreads, 3) void sgemm_kernel(const SgemmArgs g0,
         if (mirror) g.C[(size_t)col * g.ldc + row] = out;
       }
     }
+}
+
+template <bool TA, bool TB>
+__global__ __launch_bounds__(kGThreads, 3) void sgemm_kernel(const SgemmArgs g0, const Batch bt, const unsigned where) {
+  SgemmArgs g = g0;
+  if (bt.n > 1) {
+    const int z = blockIdx.z;
+    g.A = shifted(g0.A, where & kAInWs ? bt.dws[z] : bt.dq[z]);
+    g.B = shifted(g0.B, where & kBInWs ? bt.dws[z] : bt.dq[z]);
+    g.C = shifted(g0.C, where & kCInWs ? bt.dws[z] : bt.dq[z]);
+    if (g0.part) g.part = shifted(g0.part, bt.dws[z]);
+  }
+  sgemm_tile<TA, TB>(g, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+// Several independent products of one orientation in one launch: workgroup b belongs to the problem whose range of tiles holds b.
+// The products of SOAP on a model of many mid-sized matrices (a 768 x 2304 projection is 108 tiles) leave most of the chip idle one
+// at a time; together they fill it.  The tile body is the one of sgemm_kernel, so a product's bits do not depend on its company.
+constexpr int kMaxGroup = 40;
+struct SgemmGroup {
+  SgemmArgs it[kMaxGroup];
+  int tile_begin[kMaxGroup + 1];
+  int n;
+};
+static_assert(sizeof(SgemmGroup) <= 4096, "the group travels as a kernel argument");
+template <bool TA, bool TB>
+__global__ __launch_bounds__(kGThreads, 3) void sgemm_group_kernel(const SgemmGroup grp) {
+  typedef const __attribute__((address_space(4))) SgemmGroup* group_ptr_t;
+  const group_ptr_t ka = (group_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+  int lo = 0, hi = ka->n - 1;  // the last problem whose first tile is not past this workgroup
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int)blockIdx.x >= ka->tile_begin[mid]) lo = mid;
+    else hi = mid - 1;
+  }
+  SgemmArgs g;
+  g.A = ka->it[lo].A; g.B = ka->it[lo].B; g.C = ka->it[lo].C;
+  g.M = ka->it[lo].M; g.N = ka->it[lo].N; g.K = ka->it[lo].K;
+  g.lda = ka->it[lo].lda; g.ldb = ka->it[lo].ldb; g.ldc = ka->it[lo].ldc;
+  g.accumulate = ka->it[lo].accumulate; g.alpha_acc = ka->it[lo].alpha_acc; g.beta_c = ka->it[lo].beta_c;
+  g.k_chunk = 0; g.part = nullptr; g.sym = 0;
+  sgemm_tile<TA, TB>(g, (int)blockIdx.x - ka->tile_begin[lo], 0);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -876,6 +911,59 @@ extern "C" int hb_gemm_f32(const float* A, const float* B, float* C, int64_t M, 
     else sgemm_kernel<false, false><<<(unsigned)tiles, kGThreads, 0, s>>>(g, Batch{}, 0u);
   }
   return check_launch("hb_gemm_f32");
+}
+
+extern "C" int hb_gemm_f32_grouped(int32_t n, const float* const* A, const float* const* B, float* const* C, const int64_t* M, const int64_t* N,
+                                   const int64_t* K, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, int32_t trans_a, int32_t trans_b,
+                                   const int32_t* accumulate, const float* alpha_acc, const float* beta_c, void* stream_) {
+  using namespace hb;
+  if (n < 0) return set_error(HB_EINVAL, "hb_gemm_f32_grouped: negative count");
+  if (n == 0) return HB_OK;
+  if (!A || !B || !C || !M || !N || !K || !lda || !ldb || !ldc || !accumulate || !alpha_acc || !beta_c)
+    return set_error(HB_EINVAL, "hb_gemm_f32_grouped: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream_);
+  SgemmGroup grp;
+  grp.n = 0;
+  grp.tile_begin[0] = 0;
+  auto flush = [&]() {
+    if (grp.n == 0) return;
+    const unsigned blocks = (unsigned)grp.tile_begin[grp.n];
+    if (trans_a) {
+      if (trans_b) sgemm_group_kernel<true, true><<<blocks, kGThreads, 0, s>>>(grp);
+      else sgemm_group_kernel<true, false><<<blocks, kGThreads, 0, s>>>(grp);
+    } else {
+      if (trans_b) sgemm_group_kernel<false, true><<<blocks, kGThreads, 0, s>>>(grp);
+      else sgemm_group_kernel<false, false><<<blocks, kGThreads, 0, s>>>(grp);
+    }
+    grp.n = 0;
+  };
+  for (int i = 0; i < n; ++i) {
+    if (!A[i] || !B[i] || !C[i]) return set_error(HB_EINVAL, "hb_gemm_f32_grouped: null matrix pointer at %d", i);
+    if (M[i] <= 0 || N[i] <= 0 || K[i] <= 0 || M[i] > (1 << 24) || N[i] > (1 << 24) || K[i] > (1 << 24))
+      return set_error(HB_EINVAL, "hb_gemm_f32_grouped: bad shape at %d", i);
+    const int64_t big_tiles = (M[i] / kBM) * (N[i] / kBN);
+    const bool big = M[i] % kBM == 0 && N[i] % kBN == 0 && K[i] % kBK == 0 && lda[i] % 4 == 0 && ldb[i] % 4 == 0 && ldc[i] >= N[i] &&
+                     ((reinterpret_cast<uintptr_t>(A[i]) | reinterpret_cast<uintptr_t>(B[i])) & 15) == 0 && big_tiles >= sgemm_big_min_tiles();
+    const int64_t tiles = ((M[i] + kGM - 1) / kGM) * ((N[i] + kGN - 1) / kGN);
+    if (big || tiles > (1 << 22)) {  // fills the chip on its own: the single call's kernels (and its checks)
+      if (int rc = hb_gemm_f32(A[i], B[i], C[i], M[i], N[i], K[i], lda[i], ldb[i], ldc[i], trans_a, trans_b, accumulate[i], alpha_acc[i], beta_c[i],
+                               stream_))
+        return rc;
+      continue;
+    }
+    const int64_t need_a = trans_a ? M[i] : K[i], need_b = trans_b ? K[i] : N[i];
+    if (lda[i] < need_a || ldb[i] < need_b || ldc[i] < N[i]) return set_error(HB_EINVAL, "hb_gemm_f32_grouped: leading dimension too small at %d", i);
+    if (accumulate[i] & ~(HB_GEMM_ACCUMULATE | HB_GEMM_SYMMETRIC)) return set_error(HB_EINVAL, "hb_gemm_f32_grouped: unknown flag at %d", i);
+    if ((accumulate[i] & HB_GEMM_SYMMETRIC) && !(A[i] == B[i] && lda[i] == ldb[i] && M[i] == N[i] && (trans_a != 0) != (trans_b != 0)))
+      return set_error(HB_EINVAL, "hb_gemm_f32_grouped: HB_GEMM_SYMMETRIC takes one matrix as both operands, transposed on exactly one side (%d)", i);
+    if (grp.n == kMaxGroup || (int64_t)grp.tile_begin[grp.n] + tiles > 0x3FFFFFFF) flush();
+    grp.it[grp.n] = SgemmArgs{A[i], B[i], C[i], (int)M[i], (int)N[i], (int)K[i], (int)lda[i], (int)ldb[i], (int)ldc[i],
+                              accumulate[i] & HB_GEMM_ACCUMULATE, alpha_acc[i], beta_c[i], 0, nullptr, 0};
+    grp.tile_begin[grp.n + 1] = grp.tile_begin[grp.n] + (int)tiles;
+    ++grp.n;
+  }
+  flush();
+  return check_launch("hb_gemm_f32_grouped");
 }
 
 extern "C" int hb_adam_precond(float* exp_avg, float* exp_avg_sq, const float* grad, float* out, int64_t n, float a1, float one_minus_a1, float a2,

@@ -28,6 +28,7 @@ import torch
 from . import _lib
 from .optim import HBOptimizer, _ECC_DTYPES, _PLAIN_FMT, beta_debias, build_defaults, current_stream_ptr, debiased_weights, f32, mars_weights, use_default
 
+_GGT_CHUNK = 4096  # rows per independent piece of a long tensor's factor update (SOAP._update_ggt)
 K_OLD = "mars_mars_old_grad_5"  # MARS' guard, three places behind the transform's in the reference's index walk
 K_M, K_V, K_Q, K_GG = "scale_by_soap_exp_avg_2", "scale_by_soap_exp_avg_sq_2", "scale_by_soap_Q_3", "scale_by_soap_GG_3"
 
@@ -71,19 +72,76 @@ def split_blocks(shape, max_precond_dim: int):
 
 
 class _Gemm:
-    """Thin caller of hb_gemm_f32 on contiguous 2-D fp32 tensors."""
+    """Thin caller of hb_gemm_f32 on contiguous 2-D fp32 tensors.
+
+    Between ``defer()`` and ``stop()`` the products are collected instead of launched, and ``flush()`` issues them through
+    hb_gemm_f32_grouped: the products of different tensors (``owner``) are independent and share launches, the n-th product
+    asked for on behalf of one owner since the last flush runs after that owner's (n-1)-th.  Nothing but another collected
+    product may read a collected product's result before the flush."""
 
     def __init__(self, device):
         self.L = _lib.lib()
         self.device = device
+        self.queue = None  # level -> [(A, B, C, M, N, K, ta, tb, flags, alpha, beta)] while deferring
+        self.owner = None
+        self._level: Dict[object, int] = {}
+        self._then: List = []
 
-    def __call__(self, A, B, C, ta=False, tb=False, accumulate=False, alpha=1.0, beta=0.0, symmetric=False):
+    def defer(self):
+        self.queue, self._level = {}, {}
+
+    def then(self, fn):
+        """Runs ``fn`` once the products asked for so far have been issued: at once, or after the next flush while deferring."""
+        if self.queue is None:
+            fn()
+        else:
+            self._then.append(fn)
+
+    def stop(self):
+        self.flush()
+        self.queue = None
+
+    def flush(self):
+        if not self.queue and not self._then:
+            return
+        stream = current_stream_ptr(self.device)
+        for level in sorted(self.queue):
+            by_orientation: Dict[tuple, List] = {}
+            for call in self.queue[level]:
+                by_orientation.setdefault((call[6], call[7]), []).append(call)
+            for (ta, tb), calls in by_orientation.items():
+                n = len(calls)
+                ptr = lambda k: (ctypes.c_void_p * n)(*[c[k].data_ptr() for c in calls])  # noqa: E731
+                i64 = lambda vals: (ctypes.c_int64 * n)(*vals)  # noqa: E731
+                _lib.check(self.L.hb_gemm_f32_grouped(n, ptr(0), ptr(1), ptr(2), i64([c[3] for c in calls]), i64([c[4] for c in calls]),
+                                                      i64([c[5] for c in calls]), i64([c[0].shape[1] for c in calls]),
+                                                      i64([c[1].shape[1] for c in calls]), i64([c[4] for c in calls]), int(ta), int(tb),
+                                                      (ctypes.c_int32 * n)(*[c[8] for c in calls]), (ctypes.c_float * n)(*[c[9] for c in calls]),
+                                                      (ctypes.c_float * n)(*[c[10] for c in calls]), stream), "hb_gemm_f32_grouped")  # fmt: skip
+        self.queue, self._level = {}, {}
+        hooks, self._then = self._then, []
+        for fn in hooks:
+            fn()
+
+    def barrier(self):
+        """What the current owner asks for next waits for everything it has asked for so far (``independent`` products included)."""
+        if self.queue is not None:
+            self._level[self.owner] = self._level.get(self.owner, 0) + 1
+
+    def __call__(self, A, B, C, ta=False, tb=False, accumulate=False, alpha=1.0, beta=0.0, symmetric=False, independent=False):
+        """``independent``: the product neither reads nor overwrites what the owner's last product wrote, and may share its launch."""
         M = A.shape[1] if ta else A.shape[0]
         K = A.shape[0] if ta else A.shape[1]
         N = B.shape[0] if tb else B.shape[1]
         assert (B.shape[1] if tb else B.shape[0]) == K and tuple(C.shape) == (M, N)
         assert A.is_contiguous() and B.is_contiguous() and C.is_contiguous() and A.dtype == B.dtype == C.dtype == torch.float32
         flags = (_lib.GEMM_ACCUMULATE if accumulate else 0) | (_lib.GEMM_SYMMETRIC if symmetric else 0)
+        if self.queue is not None:
+            level = self._level.get(self.owner, 0)
+            if not independent:
+                self._level[self.owner] = level + 1
+            self.queue.setdefault(level, []).append((A, B, C, M, N, K, ta, tb, flags, alpha, beta))
+            return C
         _lib.check(self.L.hb_gemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.shape[1], B.shape[1], N, int(ta), int(tb),
                                       flags, alpha, beta, current_stream_ptr(self.device)), "hb_gemm_f32")  # fmt: skip
         return C
@@ -395,6 +453,69 @@ class SOAP(HBOptimizer):
                             refresh.append((GG, Q, self._widen(L, st, K_M, mom_fmt, stream), st, base))
                     return True
 
+                # Tensors beyond their first step whose view has at most two dimensions go through the preconditioner stage by
+                # stage, all of them together, so that each stage's products share launches (hb_gemm_f32_grouped): on a model of
+                # many mid-sized matrices one product at a time leaves most of the chip idle.  The arithmetic per tensor is that of
+                # ``precondition``.  A batch ends when its temporaries reach a quarter of a GiB-element.
+                staged: List[dict] = []
+
+                def run_staged():
+                    if not staged:
+                        return
+                    gemm.defer()
+                    for w in staged:  # into the eigenbasis
+                        gemm.owner = id(w)
+                        w["GG"], w["Q"] = self._factors32(w["st"])
+                        w["gp"] = self._project(gemm, w["G"], w["Q"], back=False)
+                    gemm.flush()
+                    a1, oma1 = debiased_weights(beta1, adam_step)
+                    a2, oma2 = debiased_weights(beta2, adam_step)
+                    for w in staged:  # Adam there
+                        st, gp = w["st"], w["gp"]
+                        if gp is w["G"]:
+                            gp = w["gp"] = w["G"].clone()
+                        m32, v32 = self._widen(L, st, K_M, mom_fmt, stream), self._widen(L, st, K_V, mom_fmt, stream)
+                        _lib.check(L.hb_adam_precond(m32.data_ptr(), v32.data_ptr(), gp.data_ptr(), gp.data_ptr(), gp.numel(), a1, oma1,
+                                                     a2, oma2, float(f32(group["eps"])), stream), "hb_adam_precond")  # fmt: skip
+                        if mom_fmt != _lib.FMT_F32:
+                            self._narrow(L, st, K_M, m32, mom_fmt, _lib.STREAM_EXP_AVG, step, w["base"], stream)
+                            self._narrow(L, st, K_V, v32, mom_fmt, _lib.STREAM_EXP_AVG_SQ, step, w["base"], stream)
+                    for w in staged:  # and back
+                        gemm.owner = id(w)
+                        w["back"] = self._project(gemm, w["gp"], w["Q"], back=True, out=w["out"])
+                    gemm.flush()
+                    sb = beta_debias(group["shampoo_beta"], step)  # heavyball/chainable.py:1244: python float and int64 0-d tensor
+                    a = 1 - sb
+                    a = a.to(torch.float32) if isinstance(a, torch.Tensor) else f32(a)
+                    for w in staged:  # the factors take the update's outer products
+                        if w["back"] is not w["out"]:
+                            w["out"].copy_(w["back"])
+                        gemm.owner = id(w)
+                        self._update_ggt(gemm, w["G"], w["GG"], float(a), float(1 - a))
+                    gemm.stop()
+                    for w in staged:
+                        st = w["st"]
+                        self._store_factors(L, st, K_GG, w["GG"], _lib.STREAM_SOAP_GG, step, w["base"], stream)
+                        if is_precond:
+                            exp_avg = st[K_M] if mom_fmt == _lib.FMT_F32 else self._widen(L, st, K_M, mom_fmt, stream)
+                            refresh.append((w["GG"], w["Q"], exp_avg, st, w["base"]))
+                        if w["after"] is not None:
+                            w["after"]()
+                    staged.clear()
+
+                def take(st, G0, G, out, base, fdt, after):
+                    """One tensor or block on its way through the preconditioner, staged with the others where that is possible;
+                    ``after`` runs once its update is in ``out``.  False on the first step, which only initialises."""
+                    if K_M not in st or G.dim() > 2 or not self.group_products:
+                        done = precondition(st, G0, G, out, base, fdt)
+                        if done and after is not None:
+                            after()
+                        return done
+                    staged.append(dict(st=st, G=G, out=out, base=base, after=after))
+                    if sum(w["G"].numel() for w in staged) >= 1 << 28:
+                        run_staged()
+                    return True
+
                 for (i, p, g), g32, gdt in zip(items, raw[key], gdts[key]):
                     keep.append(g32)
                     # heavyball/utils.py:3726-3742: without merge_dims the parameter is taken as it is
@@ -411,7 +532,7 @@ class SOAP(HBOptimizer):
                     out = b.slab.view("_update", i).view(G.shape)
                     blocks = split_blocks(p.shape, max_dim) if merging and group.get("split") and p.dim() > 0 else None
                     if blocks is None:
-                        if precondition(self._state0(p), G0, G, out, int(b.slab.offsets_np[i]), gdt):
+                        if take(self._state0(p), G0, G, out, int(b.slab.offsets_np[i]), gdt, None):
                             updated.append(i)
                         continue
                     # split: every block is preconditioned on its own, with its own state (heavyball/utils.py:274-286, :1612-1623);
@@ -422,12 +543,13 @@ class SOAP(HBOptimizer):
                         g0b = G0[where].contiguous().reshape(bshape)
                         gb = g0b if G is G0 else G[where].contiguous().reshape(bshape)
                         ob = torch.empty_like(gb)
-                        if precondition(self.state[p].setdefault(k, {}), g0b, gb, ob, start, gdt):
-                            out[where].copy_(ob.reshape(out[where].shape))
+                        scatter = lambda ob=ob, where=where, out=out: out[where].copy_(ob.reshape(out[where].shape))  # noqa: E731
+                        if take(self.state[p].setdefault(k, {}), g0b, gb, ob, start, gdt, scatter):
                             done = True
                         start += gb.numel()
                     if done:
                         updated.append(i)
+                run_staged()
                 if first:
                     for (st, *_), Q in zip(first, self._first_bases_of([e[1:] for e in first])):
                         st[K_Q] = Q
@@ -685,11 +807,30 @@ class SOAP(HBOptimizer):
         for d, m in enumerate(GG):  # a vector has a factor only under precondition_1d, a scalar never
             if m is None:
                 continue
-            if d == G.dim() - 1:
-                X = G.reshape(-1, G.shape[-1])
+            last = d == G.dim() - 1
+            X = G.reshape(-1, G.shape[-1]) if last else (G if d == 0 else G.movedim(d, 0).contiguous()).reshape(G.shape[d], -1)
+            depth, width = (X.shape[0], X.shape[1]) if last else (X.shape[1], X.shape[0])
+            if last and depth >= 4 * _GGT_CHUNK and ((width + 127) // 128) ** 2 < 128:
+                # a small factor of a very long tensor (an embedding's: 768 x 768 from 50257 rows) is a handful of tiles with
+                # thousands of steps each: the rows are cut into chunks whose products are independent (they share a launch),
+                # added up in chunk order and folded into the factor with the product kernel's own arithmetic,
+                # m * (1 - a) + sum * a, every operation rounded once
+                cuts = list(range(0, depth, _GGT_CHUNK))
+                parts = torch.empty((len(cuts), width, width), dtype=torch.float32, device=G.device)
+                for c, k0 in enumerate(cuts):
+                    Xc = X[k0 : k0 + _GGT_CHUNK]
+                    gemm(Xc, Xc, parts[c], ta=True, symmetric=True, independent=True)
+                gemm.barrier()
+
+                def fold(m=m, parts=parts):
+                    total = parts.sum(dim=0)
+                    total.mul_(a)
+                    m[0].mul_(one_minus_a).add_(total)
+
+                gemm.then(fold)
+            elif last:
                 gemm(X, X, m[0], ta=True, accumulate=True, alpha=a, beta=one_minus_a, symmetric=True)
             else:
-                X = (G if d == 0 else G.movedim(d, 0).contiguous()).reshape(G.shape[d], -1)
                 gemm(X, X, m[0], tb=True, accumulate=True, alpha=a, beta=one_minus_a, symmetric=True)
 
     def _refresh(self, gemm, jobs):
@@ -780,6 +921,10 @@ class SOAP(HBOptimizer):
             jobs[pi][2][0].copy_(E)
         for sd in sides:
             sd["q"][0].copy_(sd["new_q"])
+
+    #: let the products of different tensors share launches (hb_gemm_f32_grouped); False runs every tensor on its own, one product
+    #: after the other, which tests use to compare the two routes
+    group_products = True
 
     def _ortho_streams(self, dev, n: int):
         pool = self.__dict__.setdefault("_side_streams", {}).setdefault(dev, [])

@@ -30,7 +30,7 @@ extern "C" {
 
 /* Raised whenever a struct layout, an enum value or a signature changes.  A binding records the value it was written
  * against and compares it with hb_abi_version() after loading the library. */
-#define HB_ABI_VERSION 11
+#define HB_ABI_VERSION 12
 
 /* Elements per work chunk.  Every tensor starts at a slab offset that is a multiple of this, and a chunk never
  * spans two tensors. */
@@ -346,6 +346,16 @@ int hb_ns_product(int32_t tile, int32_t mode, const void* A, const void* B, void
 int hb_gemm_f32(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                 int64_t ldc, int32_t trans_a, int32_t trans_b, int32_t accumulate, float alpha_acc, float beta_c,
                 void* stream);
+/* n independent hb_gemm_f32 products of one orientation in as few launches as possible (HOST arrays of n entries; A, B, C
+ * hold device pointers): the counterpart in the reference is the loop over a group's tensors around project / update_ggt
+ * (heavyball/chainable.py:1257-1275).  A product that fills the GPU on its own runs as hb_gemm_f32 would run it; the others
+ * share launches, every workgroup finding its product in a table, so that the mid-sized products of a model with many
+ * matrices (108 tiles for a 768 x 2304 projection) fill the chip together.  Every product's result is bit-identical to its
+ * own hb_gemm_f32 call.  The products must not depend on each other. */
+int hb_gemm_f32_grouped(int32_t n, const float* const* A, const float* const* B, float* const* C, const int64_t* M,
+                        const int64_t* N, const int64_t* K, const int64_t* lda, const int64_t* ldb, const int64_t* ldc,
+                        int32_t trans_a, int32_t trans_b, const int32_t* accumulate, const float* alpha_acc,
+                        const float* beta_c, void* stream);
 int hb_adam_precond(float* exp_avg, float* exp_avg_sq, const float* grad, float* out, int64_t n, float a1,
                     float one_minus_a1, float a2, float one_minus_a2, float eps, void* stream);
 

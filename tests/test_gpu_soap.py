@@ -407,6 +407,118 @@ def test_soap_first_bases_of_several_tensors_are_found_together():
     assert sorted(widths) == sorted([96, 256, 300, 96, 96, 96, 64, 200, 6, 40, 50])
 
 
+@pytest.mark.parametrize("kwargs", [dict(precondition_frequency=3, weight_decay=0.01), dict(precondition_frequency=2, ecc="bf16+8", caution=True),
+                                    dict(precondition_frequency=3, split=True, max_precond_dim=64, mars=True)])
+def test_soap_grouped_products_equal_one_by_one(kwargs):
+    """The staged route (every stage's products of all tensors in shared launches, hb_gemm_f32_grouped) against the route that
+    takes one tensor after the other: the same tile body adds the same terms in the same order, so parameters, moments, factors
+    and bases agree bit for bit over six steps with refreshes; matrices of several shapes, a vector, a stack that keeps three
+    dimensions (which stays on the one-by-one route either way) and, in the third case, tensors cut into blocks."""
+    shapes = [(96, 200), (200, 96), (96, 96), (130, 70), (33,), (6, 40, 50), (300, 520)]
+    gen = torch.Generator().manual_seed(9)
+    host = [torch.randn(s, generator=gen) * 0.02 for s in shapes]
+    pa = [torch.nn.Parameter(h.clone().to(DEV)) for h in host]
+    pb = [torch.nn.Parameter(h.clone().to(DEV)) for h in host]
+    kwargs = dict(max_precond_dim=512, **kwargs) if "max_precond_dim" not in kwargs else kwargs
+    oa, ob = heavyball_amd.SOAP(pa, **kwargs), heavyball_amd.SOAP(pb, **kwargs)
+    ob.group_products = False
+    for o in (oa, ob):
+        o.rng_seed = 31
+    print("case", kwargs, flush=True)
+    for k in range(6):
+        grads = [torch.randn(s, generator=gen) * 1e-2 for s in shapes]
+        for p, q, g in zip(pa, pb, grads):
+            p.grad, q.grad = g.to(DEV), g.to(DEV).clone()
+        oa.step()
+        ob.step()
+    torch.cuda.synchronize()
+
+    def same(a, b, where):
+        if isinstance(a, torch.Tensor):
+            assert torch.equal(a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)), where
+        elif isinstance(a, dict):
+            assert set(a) == set(b), where
+            for kk in a:
+                same(a[kk], b[kk], f"{where}/{kk}")
+        elif isinstance(a, (list, tuple)):
+            assert len(a) == len(b), where
+            for n, (x, y) in enumerate(zip(a, b)):
+                same(x, y, f"{where}[{n}]")
+        else:
+            assert a == b, where
+
+    for i, (p, q) in enumerate(zip(pa, pb)):
+        same(p.detach(), q.detach(), f"parameter {i}")
+        same(dict(oa.state[p]), dict(ob.state[q]), f"state {i}")
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_grouped_products_are_bit_identical_to_single_calls(ta, tb):
+    """hb_gemm_f32_grouped: 45 products of one orientation (more than one launch's table holds), ragged and aligned shapes, one
+    that fills the GPU on its own (and goes through the single call's big-tile kernel), some accumulating into their output:
+    every result equals the single hb_gemm_f32 call's bit for bit, and a float64 product to 1e-6."""
+    gen = torch.Generator().manual_seed(17)
+    shapes = [(96 + 8 * (k % 5), 130 + 64 * (k % 4), 70 + 16 * (k % 7)) for k in range(43)] + [(2048, 4096, 256), (1, 1, 1)]
+    calls = []
+    for k, (M, N, K) in enumerate(shapes):
+        A = (torch.randn((K, M) if ta else (M, K), generator=gen)).to(DEV)
+        B = (torch.randn((N, K) if tb else (K, N), generator=gen)).to(DEV)
+        C = torch.randn(M, N, generator=gen).to(DEV)
+        calls.append((A, B, C, k % 3 == 0))
+    print("case", ta, tb, flush=True)
+    single, grouped = _Gemm(DEV), _Gemm(DEV)
+    want = []
+    for A, B, C, acc in calls:
+        want.append(single(A, B, C.clone(), ta=ta, tb=tb, accumulate=acc, alpha=0.25, beta=0.5))
+    grouped.defer()
+    got = []
+    for k, (A, B, C, acc) in enumerate(calls):
+        grouped.owner = k
+        got.append(grouped(A, B, C.clone(), ta=ta, tb=tb, accumulate=acc, alpha=0.25, beta=0.5))
+    grouped.stop()
+    torch.cuda.synchronize()
+    for k, (w, g) in enumerate(zip(want, got)):
+        assert torch.equal(w.view(torch.int32), g.view(torch.int32)), (k, shapes[k])
+        A, B, C, acc = calls[k]
+        ref = (A.double().T if ta else A.double()) @ (B.double().T if tb else B.double())
+        ref = C.double() * 0.5 + ref * 0.25 if acc else ref
+        assert ((g.double() - ref).norm() / ref.norm().clamp(min=1e-30)).item() < 1e-6
+
+
+def test_soap_factor_update_of_a_long_tensor_in_chunks():
+    """A small factor of a very long tensor (an embedding's) is updated from independent products of 4096-row chunks, added up in
+    chunk order and folded in as m (1 - a) + sum a: against float64, and bit for bit between the immediate and the collected
+    route of the product caller (where the chunks share one launch)."""
+    from heavyball_amd import soap as S
+
+    gen = torch.Generator().manual_seed(2)
+    G = (torch.randn(20000, 200, generator=gen) * 1e-2).to(DEV)
+    m0 = torch.randn(200, 200, generator=gen)
+    m0 = (m0 @ m0.T * 1e-3).to(DEV)
+    a = 0.05
+    want = m0.double() * (1 - a) + (G.double().T @ G.double()) * a
+    outs = []
+    for collected in (False, True):
+        gemm = _Gemm(DEV)
+        GG = [None, m0.clone()[None]]
+        if collected:
+            gemm.defer()
+            gemm.owner = "t"
+        S.SOAP._update_ggt(gemm, G, GG, a, 1 - a)
+        if collected:
+            assert len(gemm.queue) == 1 and len(gemm.queue[0]) == 5  # five chunks, one level
+            gemm.stop()
+        torch.cuda.synchronize()
+        outs.append(GG[1][0].clone())
+        assert ((GG[1][0].double() - want).norm() / want.norm()).item() < 1e-6
+    assert torch.equal(outs[0], outs[1])
+    # below the length that is worth cutting: the one product with its own accumulation
+    GG = [None, m0.clone()[None]]
+    S.SOAP._update_ggt(_Gemm(DEV), G[:9000].contiguous(), GG, a, 1 - a)
+    want = m0.double() * (1 - a) + (G[:9000].double().T @ G[:9000].double()) * a
+    assert ((GG[1][0].double() - want).norm() / want.norm()).item() < 1e-6
+
+
 def test_soap_mid_size_own_eigh_signed_momentum():
     """[256, 256] and [512, 512] Gaussian gradients with the optimizer's own eigh (no basis adopted) over two refreshes:
     square gradients give full-rank factors from the first step on, so the eigenbasis is unique up to column signs, and
