@@ -118,6 +118,8 @@ _PROTOTYPES = {
     "hb_orthonormalize_f32_batched": (ctypes.c_int, [c_int32, POINTER(c_void_p), c_int64, c_int64, c_int64, POINTER(c_void_p), c_int64,
                                                      POINTER(c_void_p), c_void_p]),
     "hb_adam_precond": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_float, c_float, c_void_p]),
+    "hb_adam_precond_grouped": (ctypes.c_int, [c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64),
+                                               c_float, c_float, c_float, c_float, c_float, c_void_p]),
     "hb_copy_probe": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "hb_last_error": (c_char_p, []),
     "hb_chunk_elems": (ctypes.c_int, []),

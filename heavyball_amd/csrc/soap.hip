@@ -504,6 +504,47 @@ __global__ __launch_bounds__(256) void adam_precond_kernel(float* __restrict__ m
   }
 }
 
+// The same for several tensors in one launch: tensor t owns workgroups [block_begin[t], block_begin[t + 1]), each of which walks
+// its tensor with that many workgroups' stride (a model's vectors are a few hundred elements each: one launch per tensor is all
+// launch latency).
+constexpr int kMaxAdamGroup = 80;
+struct AdamGroup {
+  float* m[kMaxAdamGroup];
+  float* v[kMaxAdamGroup];
+  const float* g[kMaxAdamGroup];
+  float* out[kMaxAdamGroup];
+  int64_t n[kMaxAdamGroup];
+  int block_begin[kMaxAdamGroup + 1];
+  int count;
+  float a1, oma1, a2, oma2, eps;
+};
+static_assert(sizeof(AdamGroup) <= 4096, "the group travels as a kernel argument");
+__global__ __launch_bounds__(256) void adam_precond_group_kernel(const AdamGroup grp) {
+  typedef const __attribute__((address_space(4))) AdamGroup* group_ptr_t;
+  const group_ptr_t ka = (group_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+  int lo = 0, hi = ka->count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int)blockIdx.x >= ka->block_begin[mid]) lo = mid;
+    else hi = mid - 1;
+  }
+  float* __restrict__ m = ka->m[lo];
+  float* __restrict__ v = ka->v[lo];
+  const float* __restrict__ gr = ka->g[lo];
+  float* __restrict__ out = ka->out[lo];
+  const int64_t n = ka->n[lo];
+  const int first = ka->block_begin[lo], blocks = ka->block_begin[lo + 1] - first;
+  const float a1 = ka->a1, oma1 = ka->oma1, a2 = ka->a2, oma2 = ka->oma2, eps = ka->eps;
+  for (int64_t i = (int64_t)((int)blockIdx.x - first) * 256 + threadIdx.x; i < n; i += (int64_t)blocks * 256) {
+    const float x = gr[i];
+    const float mm = m[i] * oma1 + x * a1;
+    const float vv = v[i] * oma2 + (x * x) * a2;
+    m[i] = mm;
+    v[i] = vv;
+    out[i] = mm / __builtin_fmaxf(__builtin_sqrtf(vv), eps);
+  }
+}
+
 // split-K: adds the partial products in a fixed order (deterministic) and applies the epilogue of sgemm_kernel
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int splits, int M, int N, float* __restrict__ C,
                                                             int ldc, int accumulate, float alpha_acc, float beta_c, const Batch bt,
@@ -976,6 +1017,37 @@ extern "C" int hb_adam_precond(float* exp_avg, float* exp_avg_sq, const float* g
   adam_precond_kernel<<<(unsigned)(blocks > 65536 ? 65536 : blocks), 256, 0, static_cast<hipStream_t>(stream_)>>>(
       exp_avg, exp_avg_sq, grad, out, n, a1, one_minus_a1, a2, one_minus_a2, eps);
   return check_launch("hb_adam_precond");
+}
+
+extern "C" int hb_adam_precond_grouped(int32_t count, float* const* exp_avg, float* const* exp_avg_sq, const float* const* grad, float* const* out,
+                                       const int64_t* n, float a1, float one_minus_a1, float a2, float one_minus_a2, float eps, void* stream_) {
+  using namespace hb;
+  if (count < 0) return set_error(HB_EINVAL, "hb_adam_precond_grouped: negative count");
+  if (count == 0) return HB_OK;
+  if (!exp_avg || !exp_avg_sq || !grad || !out || !n) return set_error(HB_EINVAL, "hb_adam_precond_grouped: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream_);
+  AdamGroup grp;
+  grp.count = 0;
+  grp.block_begin[0] = 0;
+  grp.a1 = a1; grp.oma1 = one_minus_a1; grp.a2 = a2; grp.oma2 = one_minus_a2; grp.eps = eps;
+  auto flush = [&]() {
+    if (grp.count == 0) return;
+    adam_precond_group_kernel<<<(unsigned)grp.block_begin[grp.count], 256, 0, s>>>(grp);
+    grp.count = 0;
+  };
+  for (int t = 0; t < count; ++t) {
+    if (n[t] < 0) return set_error(HB_EINVAL, "hb_adam_precond_grouped: negative size at %d", t);
+    if (n[t] == 0) continue;
+    if (!exp_avg[t] || !exp_avg_sq[t] || !grad[t] || !out[t]) return set_error(HB_EINVAL, "hb_adam_precond_grouped: null pointer at %d", t);
+    const int64_t want = (n[t] + 255) / 256;
+    const int blocks = (int)(want > 16384 ? 16384 : want);
+    if (grp.count == kMaxAdamGroup || grp.block_begin[grp.count] + blocks > (1 << 22)) flush();
+    const int k = grp.count++;
+    grp.m[k] = exp_avg[t]; grp.v[k] = exp_avg_sq[t]; grp.g[k] = grad[t]; grp.out[k] = out[t]; grp.n[k] = n[t];
+    grp.block_begin[k + 1] = grp.block_begin[k] + blocks;
+  }
+  flush();
+  return check_launch("hb_adam_precond_grouped");
 }
 
 extern "C" int hb_orthonormalize_workspace_bytes(int64_t m, int64_t n, int64_t* bytes) {

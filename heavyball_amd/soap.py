@@ -458,6 +458,7 @@ class SOAP(HBOptimizer):
                 # many mid-sized matrices one product at a time leaves most of the chip idle.  The arithmetic per tensor is that of
                 # ``precondition``.  A batch ends when its temporaries reach a quarter of a GiB-element.
                 staged: List[dict] = []
+                staged_elems = [0]
 
                 def run_staged():
                     if not staged:
@@ -470,16 +471,22 @@ class SOAP(HBOptimizer):
                     gemm.flush()
                     a1, oma1 = debiased_weights(beta1, adam_step)
                     a2, oma2 = debiased_weights(beta2, adam_step)
-                    for w in staged:  # Adam there
+                    adam = []  # Adam there, for all of them in one launch
+                    for w in staged:
                         st, gp = w["st"], w["gp"]
-                        if gp is w["G"]:
-                            gp = w["gp"] = w["G"].clone()
-                        m32, v32 = self._widen(L, st, K_M, mom_fmt, stream), self._widen(L, st, K_V, mom_fmt, stream)
-                        _lib.check(L.hb_adam_precond(m32.data_ptr(), v32.data_ptr(), gp.data_ptr(), gp.data_ptr(), gp.numel(), a1, oma1,
-                                                     a2, oma2, float(f32(group["eps"])), stream), "hb_adam_precond")  # fmt: skip
-                        if mom_fmt != _lib.FMT_F32:
-                            self._narrow(L, st, K_M, m32, mom_fmt, _lib.STREAM_EXP_AVG, step, w["base"], stream)
-                            self._narrow(L, st, K_V, v32, mom_fmt, _lib.STREAM_EXP_AVG_SQ, step, w["base"], stream)
+                        src = gp
+                        if gp is w["G"]:  # no basis at all (a vector): Adam reads the update and writes the result where it belongs
+                            gp = w["gp"] = w["out"]
+                        w["m32"], w["v32"] = self._widen(L, st, K_M, mom_fmt, stream), self._widen(L, st, K_V, mom_fmt, stream)
+                        adam.append((w["m32"].data_ptr(), w["v32"].data_ptr(), src.data_ptr(), gp.data_ptr(), gp.numel()))
+                    n = len(adam)
+                    cols = [(ctypes.c_void_p * n)(*[t[k] for t in adam]) for k in range(4)]
+                    _lib.check(L.hb_adam_precond_grouped(n, *cols, (ctypes.c_int64 * n)(*[t[4] for t in adam]), a1, oma1, a2, oma2,
+                                                         float(f32(group["eps"])), stream), "hb_adam_precond_grouped")  # fmt: skip
+                    if mom_fmt != _lib.FMT_F32:
+                        for w in staged:
+                            self._narrow(L, w["st"], K_M, w["m32"], mom_fmt, _lib.STREAM_EXP_AVG, step, w["base"], stream)
+                            self._narrow(L, w["st"], K_V, w["v32"], mom_fmt, _lib.STREAM_EXP_AVG_SQ, step, w["base"], stream)
                     for w in staged:  # and back
                         gemm.owner = id(w)
                         w["back"] = self._project(gemm, w["gp"], w["Q"], back=True, out=w["out"])
@@ -502,6 +509,7 @@ class SOAP(HBOptimizer):
                         if w["after"] is not None:
                             w["after"]()
                     staged.clear()
+                    staged_elems[0] = 0
 
                 def take(st, G0, G, out, base, fdt, after):
                     """One tensor or block on its way through the preconditioner, staged with the others where that is possible;
@@ -512,7 +520,8 @@ class SOAP(HBOptimizer):
                             after()
                         return done
                     staged.append(dict(st=st, G=G, out=out, base=base, after=after))
-                    if sum(w["G"].numel() for w in staged) >= 1 << 28:
+                    staged_elems[0] += G.numel()
+                    if staged_elems[0] >= 1 << 28:
                         run_staged()
                     return True
 
@@ -723,12 +732,11 @@ class SOAP(HBOptimizer):
     def _project(cls, gemm, X, Q, back: bool, out=None):
         """heavyball/utils.py:1391-1411: every dimension that has a basis is rotated by it (by its transpose when ``back``).
         The last product writes into ``out`` where it can (a first or last dimension); the caller copies otherwise."""
+        dims = [d for d, q in enumerate(Q) if q is not None]
         cur = X
-        last = max((d for d, q in enumerate(Q) if q is not None), default=-1)
-        for d, q in enumerate(Q):
-            if q is not None:
-                direct = out is not None and d == last and d in (0, X.dim() - 1)
-                cur = cls._mode_product(gemm, cur, q[0], d, back, out if direct else None)
+        for d in dims:
+            direct = out is not None and d == dims[-1] and (d == 0 or d == X.dim() - 1)
+            cur = cls._mode_product(gemm, cur, Q[d][0], d, back, out if direct else None)
         return cur
 
     @staticmethod

@@ -358,6 +358,12 @@ int hb_gemm_f32_grouped(int32_t n, const float* const* A, const float* const* B,
                         const float* beta_c, void* stream);
 int hb_adam_precond(float* exp_avg, float* exp_avg_sq, const float* grad, float* out, int64_t n, float a1,
                     float one_minus_a1, float a2, float one_minus_a2, float eps, void* stream);
+/* hb_adam_precond for `count` tensors in as few launches as possible (HOST arrays of count entries holding device pointers and
+ * element counts): the vectors of a model are a few hundred elements each, and one launch per tensor is all launch latency.
+ * Elementwise, so every tensor's result is bit-identical to its own hb_adam_precond call. */
+int hb_adam_precond_grouped(int32_t count, float* const* exp_avg, float* const* exp_avg_sq, const float* const* grad,
+                            float* const* out, const int64_t* n, float a1, float one_minus_a1, float a2, float one_minus_a2,
+                            float eps, void* stream);
 
 /*
  * hb_orthonormalize_f32: Q[m, n] (row-major, leading dimension ld, n <= m) is replaced by the Q factor of its thin QR
