@@ -25,6 +25,7 @@ NS_LEGACY, NS_BF16_UPDATE, NS_F16_UPDATE, NS_APPLY_TO_PARAM, NS_CAUTIOUS_WD = 1,
 NOALLOC_MAX_TENSORS = 8192  # HB_NOALLOC_MAX_TENSORS
 CAUTION_SLOTS = 32  # HB_CAUTION_SLOTS: counters per tensor in HbStepDesc.caution_count
 GEMM_ACCUMULATE, GEMM_SYMMETRIC = 1, 2
+ORTHO_MAX_BATCH = 64  # HB_ORTHO_MAX_BATCH: matrices per hb_orthonormalize_f32_batched call
 MOM_NESTEROV_EMA, MOM_EMA, MOM_HEAVYBALL, MOM_NESTEROV_HEAVYBALL = range(4)
 
 ECC_FMT = {"bf16+8": FMT_ECC_BF16_8, "bf16+16": FMT_ECC_BF16_16, "fp16+8": FMT_ECC_F16_8, "fp16+16": FMT_ECC_F16_16}

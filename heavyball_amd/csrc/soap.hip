@@ -38,7 +38,7 @@ struct SgemmArgs {
 // Several problems of one shape in one launch (the batched orthonormalisation): the arguments describe problem 0 and
 // problem z = blockIdx.z differs only in where its matrix and its workspace lie, so every operand moves by the byte
 // distance of its home (matrix or workspace) from that of problem 0.  n <= 1: a plain launch.
-constexpr int kMaxBatch = 8;
+constexpr int kMaxBatch = HB_ORTHO_MAX_BATCH;  // Batch travels as a kernel argument beside the product's own (1.6 of 4 KiB)
 struct Batch {
   int n;
   int64_t dq[kMaxBatch];    // byte distance of matrix z from matrix 0

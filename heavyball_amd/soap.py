@@ -169,7 +169,7 @@ class _Ortho:
 
 def launch_orthonormalize(jobs: List[_Ortho], stream: Optional[torch.cuda.Stream] = None):
     """Starts the factorisations of ``jobs``: matrices of one shape go through ``hb_orthonormalize_f32_batched`` in groups of
-    up to eight (every launch of the chain then covers the whole group), the rest one by one."""
+    up to ``_lib.ORTHO_MAX_BATCH`` (every launch of the chain then covers the whole group), the rest one by one."""
     L = _lib.lib()
     groups: Dict[tuple, List[_Ortho]] = {}
     for j in jobs:
@@ -177,8 +177,8 @@ def launch_orthonormalize(jobs: List[_Ortho], stream: Optional[torch.cuda.Stream
     for (shape, dev, _), members in groups.items():
         sp = current_stream_ptr(dev) if stream is None else stream.cuda_stream
         with torch.cuda.device(dev):
-            for k in range(0, len(members), 8):
-                part = members[k : k + 8]
+            for k in range(0, len(members), _lib.ORTHO_MAX_BATCH):
+                part = members[k : k + _lib.ORTHO_MAX_BATCH]
                 if len(part) == 1:
                     part[0].launch(stream)
                     continue
@@ -870,16 +870,24 @@ class SOAP(HBOptimizer):
         streams = self._ortho_streams(dev, len(by_shape))
         for gi, width in enumerate(sorted(by_shape, reverse=True)):  # longest chains first
             ks = by_shape[width]
-            for k in ks:
+            # the sides of one width together: their GG @ Q products share launches, and the estimates, their order and the
+            # reordered columns are computed on stacked tensors (a model has dozens of bases of one width)
+            tmp_all = torch.empty((len(ks), width, width), dtype=torch.float32, device=dev)
+            gemm.defer()
+            for j, k in enumerate(ks):
+                gemm.owner = k
+                gemm(sides[k]["m"][0], sides[k]["q"][0], tmp_all[j])
+            gemm.stop()
+            if len(ks) * width * width <= 1 << 26:
+                eig_all = (torch.stack([sides[k]["q"][0] for k in ks]) * tmp_all).sum(dim=1)
+            else:  # wide bases: no second copy of them
+                eig_all = torch.stack([(sides[k]["q"][0] * tmp_all[j]).sum(dim=0) for j, k in enumerate(ks)])
+            idx_all = torch.argsort(eig_all, dim=-1, descending=True, stable=True).unsqueeze(1).expand_as(tmp_all)
+            ordered_all = tmp_all.gather(-1, idx_all)
+            basis_all = ordered_all.clone()
+            for j, k in enumerate(ks):
                 sd = sides[k]
-                q = sd["q"]
-                tmp = torch.empty_like(q[0])
-                gemm(sd["m"][0], q[0], tmp)
-                eig = (q[0] * tmp).sum(dim=0)
-                sd["idx"] = torch.argsort(eig, descending=True).unsqueeze(0).expand_as(tmp)
-                sd["ordered"] = tmp.gather(-1, sd["idx"])
-                sd["basis"] = sd["ordered"].clone()
-                sd["tmp"] = tmp
+                sd["idx"], sd["ordered"], sd["basis"], sd["tmp"] = idx_all[j], ordered_all[j], basis_all[j], tmp_all[j]
                 sd["job"] = _Ortho(sd["basis"], status[k : k + 1])
             # the bases of this width are sorted: their factorisations start together on the group's stream
             ready = torch.cuda.Event()
@@ -895,9 +903,16 @@ class SOAP(HBOptimizer):
             """The new Q (scattered back to the old column order) of the sides ``ks`` and the rotated exp_avg of their
             parameters, all in temporaries."""
             rotated: Dict[int, torch.Tensor] = {}
+            waited = None
+            gemm.defer()
             for k in ks:
                 sd = sides[k]
-                main.wait_event(sd["done"])  # the caller's stream goes no further until this factorisation is there
+                if sd["done"] is not waited:
+                    # the rotations collected so far belong to factorisations that are there: out with them, in shared launches,
+                    # before the caller's stream stops for the next factorisation
+                    gemm.flush()
+                    main.wait_event(sd["done"])
+                    waited = sd["done"]
                 new_q = torch.empty_like(sd["tmp"])
                 new_q.scatter_(-1, sd["idx"], sd["basis"])
                 sd["new_q"] = new_q
@@ -905,9 +920,15 @@ class SOAP(HBOptimizer):
                 # basis Q^T Q_new would cost 2 d^3 + 2 numel d (the order an einsum planner picks for the reference's
                 # five-operand expression, heavyball/utils.py:877-884, as well)
                 E = rotated.get(sd["param"], sd["exp_avg"][0])
+                if E.dim() > 2:  # a middle dimension is moved to the front by a copy, which must see the product before it
+                    gemm.stop()
+                gemm.owner = sd["param"]
                 E = self._mode_product(gemm, E, sd["q"][0], sd["d"], back=True)
                 E = self._mode_product(gemm, E, new_q, sd["d"], back=False)
                 rotated[sd["param"]] = E
+                if gemm.queue is None:
+                    gemm.defer()
+            gemm.stop()
             return rotated
 
         # optimistic pass: parameters whose longest factorisation is shortest first; the rotations of one parameter in

@@ -377,12 +377,15 @@ int hb_adam_precond_grouped(int32_t count, float* const* exp_avg, float* const* 
 int hb_orthonormalize_workspace_bytes(int64_t m, int64_t n, int64_t* bytes);
 int hb_orthonormalize_f32(float* Q, int64_t m, int64_t n, int64_t ld, void* workspace, int64_t workspace_bytes, int32_t* status,
                           void* stream);
-/* hb_orthonormalize_f32 for n_mats (1..8) matrices of one shape, every launch covering all of them: the counterpart of
+#define HB_ORTHO_MAX_BATCH 64
+/* hb_orthonormalize_f32 for n_mats (1..HB_ORTHO_MAX_BATCH) matrices of one shape, every launch covering all of them: the counterpart of
  * the reference's same-shape bucketing (heavyball/chainable.py:503-584) for the QR of get_orthogonal_matrix_QR.  A
  * factorisation is a chain of ~16 short dependent launches per panel, so n_mats matrices take about as long as one.
  * Q, workspace, status: HOST arrays of n_mats device pointers (each workspace of workspace_bytes >=
  * hb_orthonormalize_workspace_bytes(m, n), one status word per matrix; the matrices must agree in their address modulo
- * 16 bytes).  Results are bit-identical to n_mats calls of hb_orthonormalize_f32. */
+ * 16 bytes).  A matrix' result does not depend on the other matrices of its batch, but it may depend on their number: a
+ * panel product is split along K when the whole batch has too few workgroups to fill the GPU, and the split changes the
+ * order of the sum. */
 int hb_orthonormalize_f32_batched(int32_t n_mats, float* const* Q, int64_t m, int64_t n, int64_t ld, void* const* workspace,
                                   int64_t workspace_bytes, int32_t* const* status, void* stream);
 

@@ -60,7 +60,7 @@ def test_argument_checks_run_before_any_device_call():
     assert L.hb_gemm_f32(None, None, None, 4, 4, 4, 4, 4, 4, 0, 0, 0, 1.0, 0.0, None) == -1
     assert b"null pointer" in L.hb_last_error()
     one = (ctypes.c_void_p * 1)(16)
-    for n_mats in (0, 9):
+    for n_mats in (0, _lib.ORTHO_MAX_BATCH + 1):
         assert L.hb_orthonormalize_f32_batched(n_mats, one, 8, 4, 4, one, 1 << 20, one, None) == -1
         assert b"matrices per call" in L.hb_last_error()
     nb = ctypes.c_int64()
