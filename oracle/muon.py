@@ -10,7 +10,8 @@ once to bf16, up to the order of the accumulation, which no two backends share (
 the same operands, rounded to bf16, already ends 5e-3 away after five iterations); parity of the Newton-Schulz output is
 therefore a tolerance (2e-2 relative Frobenius), not bit equality.  PARITY OF THE
 NEWTON-SCHULZ NUMERICS IS NOT PINNED BY ANY TEST OF THE REFERENCE (none calls zeropower_*); it is pinned here by golden
-vectors written from the reference (tests/golden/ns5.pt) and by the polar-factor invariant.
+vectors written from the reference (tests/golden/ns5.pt; ns5_bf16.pt and ns5_fp16.pt for 16-bit update buffers; msign.pt for the
+ten-step schedule) and by the polar-factor invariant.
 """
 
 from typing import List
